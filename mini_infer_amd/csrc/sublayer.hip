@@ -1,0 +1,500 @@
+// Kernels around sublayers that add their own normed output to the residual stream, and the
+// mixers and activations that go with them:
+//   embed_sinusoid      table row * scale + interleaved sin/cos of the position -> float32 stream
+//   norm_scale_add      stream += y * rsqrt(mean(y^2) + eps) * gain * scale[c]   (norm on a sublayer's OUTPUT)
+//   cast_rows           the stream in the compute dtype, for the products that read it
+//   gated_scan          minGRU: a gated recurrence whose gates read the current token only
+//   qk_norm_kv_write    RMS norm of q and of k over the WHOLE projection; normed k -> key pages,
+//                       k as projected -> value pages (values that are the keys)
+//   poly_norm           a N(z) + b N(z^2) + c N(z^3) + e over a token's feed-forward values
+//   gated_table_rows    gelu_tanh(gate) * (a slice of a per-token table row)
+// Storage is float32 or bfloat16.  Statistics, gates, the recurrent state and the stream are
+// float32 with bfloat16 elements; with float32 elements (the 32-bit path) they are evaluated
+// in 64-bit and rounded once, as in the other per-token kernels.
+#include "common.h"
+
+#include <math.h>
+
+template <typename T>
+struct Wide {
+  using type = float;
+};
+template <>
+struct Wide<float> {
+  using type = double;
+};
+
+__device__ __forceinline__ float lane_xor(float v, int off) { return __shfl_xor(v, off, MI_WAVE); }
+__device__ __forceinline__ double lane_xor(double v, int off) { return __shfl_xor(v, off, MI_WAVE); }
+
+// Sum over the block in a fixed order; `scratch` holds one value per wave.  All threads get it.
+template <typename A>
+__device__ __forceinline__ A block_total(A v, A* scratch) {
+#pragma unroll
+  for (int off = MI_WAVE / 2; off > 0; off >>= 1) v += lane_xor(v, off);
+  const int wave = threadIdx.x / MI_WAVE, lane = threadIdx.x % MI_WAVE;
+  const int n_waves = (blockDim.x + MI_WAVE - 1) / MI_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  A total = 0;
+  for (int w = 0; w < n_waves; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float inv_root(float mean_sq, float eps) { return 1.0f / sqrtf(mean_sq + eps); }
+__device__ __forceinline__ double inv_root(double mean_sq, double eps) { return 1.0 / sqrt(mean_sq + eps); }
+__device__ __forceinline__ float logistic(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ double logistic(double z) { return 1.0 / (1.0 + exp(-z)); }
+__device__ __forceinline__ float tanh_of(float z) { return tanhf(z); }
+__device__ __forceinline__ double tanh_of(double z) { return tanh(z); }
+
+// ---------------------------------------------------------------------------
+// embedding with a scale and an added sinusoid: column 2i gets sin(p * f_i), column 2i+1
+// cos(p * f_i); `freq` [ceil(hidden/2)] holds f_i in 64-bit (made on the host).  bfloat16
+// tables take the angle in float32; the 32-bit path takes it in 64-bit.
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_sinusoid_kernel(
+    const T* __restrict__ table, const int* __restrict__ ids, const int* __restrict__ positions,
+    const double* __restrict__ freq, float* __restrict__ residual, T* __restrict__ cast, int hidden, float scale) {
+  using A = typename Wide<T>::type;
+  const int t = blockIdx.x;
+  const T* row = table + (int64_t)ids[t] * hidden;
+  const A pos = (A)positions[t];
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const A angle = pos * (A)freq[i / 2];
+    A wave;
+    if constexpr (sizeof(T) == 4) wave = (i & 1) ? cos(angle) : sin(angle);
+    else wave = (i & 1) ? cosf(angle) : sinf(angle);
+    const float v = (float)((A)to_f32(row[i]) * (A)scale + wave);
+    residual[(int64_t)t * hidden + i] = v;
+    if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(v);
+  }
+}
+
+extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, const int* positions,
+                                 const double* freq, float* residual, void* cast, int num_tokens, int hidden,
+                                 int vocab, float scale, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0, "embed_sinusoid: bad sizes tokens=%d hidden=%d vocab=%d",
+             num_tokens, hidden, vocab);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_sinusoid: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    embed_sinusoid_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)table, ids, positions, freq, residual,
+                                                                 (float*)cast, hidden, scale);
+  } else {
+    embed_sinusoid_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, positions, freq,
+                                                                  residual, (bf16_t*)cast, hidden, scale);
+  }
+  MI_CHECK_LAUNCH("embed_sinusoid");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The norm on a sublayer's output with the add folded in:
+//   residual[t, c] += y[t, c] * rsqrt(mean_c(y[t]^2) + eps) * gain * scale[c]
+// `gain` is one number or absent, `scale` one number per column or absent (both float32).
+// With `cast`, the new residual row is also written in the element type, which is what the
+// next sublayer's products read.  One block a row.
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void norm_scale_add_kernel(
+    const T* __restrict__ y, int64_t y_stride, float* __restrict__ residual, const float* __restrict__ gain,
+    const float* __restrict__ scale, T* __restrict__ cast, int hidden, float eps) {
+  using A = typename Wide<T>::type;
+  __shared__ A scratch[4];
+  const int t = blockIdx.x;
+  const T* row = y + (int64_t)t * y_stride;
+  A squares = 0;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const A v = (A)to_f32(row[i]);
+    squares += v * v;
+  }
+  const A inv = inv_root(block_total<A>(squares, scratch) / (A)hidden, (A)eps);
+  const A g = gain != nullptr ? (A)gain[0] : (A)1;
+  float* res = residual + (int64_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    A v = ((A)to_f32(row[i]) * inv) * g;
+    if (scale != nullptr) v *= (A)scale[i];
+    const float sum = (float)((A)res[i] + v);
+    res[i] = sum;
+    if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(sum);
+  }
+}
+
+extern "C" int mi_norm_scale_add(int dtype, const void* y, int64_t y_stride, float* residual, const float* gain,
+                                 const float* scale, void* cast, int num_tokens, int hidden, float eps,
+                                 hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && hidden > 0 && y_stride >= hidden, "norm_scale_add: bad sizes tokens=%d hidden=%d stride=%lld",
+             num_tokens, hidden, (long long)y_stride);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "norm_scale_add: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    norm_scale_add_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, y_stride, residual, gain, scale,
+                                                                 (float*)cast, hidden, eps);
+  } else {
+    norm_scale_add_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, y_stride, residual, gain, scale,
+                                                                  (bf16_t*)cast, hidden, eps);
+  }
+  MI_CHECK_LAUNCH("norm_scale_add");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The float32 stream in bfloat16.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void cast_rows_kernel(const float* __restrict__ in, bf16_t* __restrict__ out, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = (bf16_t)in[i];
+}
+
+extern "C" int mi_cast_rows(const float* in, void* out, int64_t n, hipStream_t stream) {
+  MI_REQUIRE(n >= 0, "cast_rows: bad size %lld", (long long)n);
+  if (n == 0) return MI_OK;
+  cast_rows_kernel<<<(unsigned)ceil_div64(n, 256), 256, 0, stream>>>(in, (bf16_t*)out, n);
+  MI_CHECK_LAUNCH("cast_rows");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// minGRU.  Row t of `zxg` holds the three projections of the token [z | x | g], `width` each.
+//   z = sigmoid(z_in + bz)          u = x_in + bx
+//   cand = u + 1/2 (u >= 0), sigmoid(u) (u < 0)
+//   S = (1 - z) * S + z * cand      out = S * silu(g)
+// S is one float32 row per state slot; request b's row is state[slots[b]] (a slot outside
+// 0..num_slots-1, the -1 of a padding row, means the spare row at index num_slots).  Request
+// b owns rows cu[b]..cu[b+1]-1; a request without rows is left alone.
+//
+// Sequential form: one thread per (request, column) walks the request's rows.
+// ---------------------------------------------------------------------------
+
+template <typename A>
+__device__ __forceinline__ void gru_gates(A z_in, A u, A& keep, A& add) {
+  const A z = logistic(z_in);
+  const A cand = u >= (A)0 ? u + (A)0.5 : logistic(u);
+  keep = (A)1 - z;
+  add = z * cand;
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void gated_scan_kernel(
+    const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
+    float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ out,
+    int64_t out_stride, int width, int num_slots) {
+  using A = typename Wide<T>::type;
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int first = cu[b], last = cu[b + 1];
+  if (last <= first) return;
+  const int slot = slots[b];
+  const int64_t row = (slot < 0 || slot >= num_slots) ? num_slots : slot;
+  A s = (A)state[row * width + c];
+  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
+#pragma unroll 4
+  for (int t = first; t < last; ++t) {
+    const T* in = zxg + (int64_t)t * in_stride;
+    const A z_in = (A)to_f32(in[c]) + bias_z;
+    const A u = (A)to_f32(in[width + c]) + bias_x;
+    const A g = (A)to_f32(in[2 * (int64_t)width + c]);
+    A keep, add;
+    gru_gates<A>(z_in, u, keep, add);
+    s = keep * s + add;
+    out[(int64_t)t * out_stride + c] = from_f32<T>((float)(s * (g * logistic(g))));
+  }
+  state[row * width + c] = (float)s;
+}
+
+// Chunked form for long portions: the recurrence S' = keep * S + add is linear in S, so a
+// chunk of rows acts on its incoming state as S_out = P * S_in + Q with P the product of its
+// keeps and Q its result from a zero state.  Pass 1 computes (P, Q) of every chunk, pass 2
+// walks each request's chunks in order and leaves every chunk's incoming state, pass 3 redoes
+// every chunk from its incoming state and writes the outputs.  Chunks are cut per request
+// at multiples of `chunk` rows from the request's first row of the step.
+template <typename T>
+__global__ __launch_bounds__(64) void gated_scan_summaries_kernel(
+    const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
+    const int* __restrict__ cu, float* __restrict__ summaries, int width, int chunk, int chunks_per_request) {
+  using A = typename Wide<T>::type;
+  const int b = blockIdx.z, k = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int first = cu[b] + k * chunk, last = min(cu[b + 1], first + chunk);
+  if (last <= first) return;
+  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
+  A p = 1, q = 0;
+#pragma unroll 4
+  for (int t = first; t < last; ++t) {
+    const T* in = zxg + (int64_t)t * in_stride;
+    A keep, add;
+    gru_gates<A>((A)to_f32(in[c]) + bias_z, (A)to_f32(in[width + c]) + bias_x, keep, add);
+    p *= keep;
+    q = keep * q + add;
+  }
+  float* at = summaries + (((int64_t)b * chunks_per_request + k) * 2) * width;
+  at[c] = (float)p;
+  at[width + c] = (float)q;
+}
+
+// Pass 2: every chunk's (P, Q) is replaced by its incoming state (in Q's place); the request's
+// state row receives the state after its last row.
+__global__ __launch_bounds__(64) void gated_scan_carry_kernel(
+    float* __restrict__ summaries, float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ slots, int width, int chunk, int chunks_per_request, int num_slots) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int rows = cu[b + 1] - cu[b];
+  if (rows <= 0) return;
+  const int slot = slots[b];
+  const int64_t row = (slot < 0 || slot >= num_slots) ? num_slots : slot;
+  const int chunks = (rows + chunk - 1) / chunk;
+  float s = state[row * width + c];
+  for (int k = 0; k < chunks; ++k) {
+    float* at = summaries + (((int64_t)b * chunks_per_request + k) * 2) * width;
+    const float p = at[c], q = at[width + c];
+    at[width + c] = s;
+    s = p * s + q;
+  }
+  state[row * width + c] = s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void gated_scan_outputs_kernel(
+    const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
+    const int* __restrict__ cu, const float* __restrict__ summaries, T* __restrict__ out, int64_t out_stride,
+    int width, int chunk, int chunks_per_request) {
+  using A = typename Wide<T>::type;
+  const int b = blockIdx.z, k = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int first = cu[b] + k * chunk, last = min(cu[b + 1], first + chunk);
+  if (last <= first) return;
+  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
+  A s = (A)summaries[(((int64_t)b * chunks_per_request + k) * 2 + 1) * width + c];
+#pragma unroll 4
+  for (int t = first; t < last; ++t) {
+    const T* in = zxg + (int64_t)t * in_stride;
+    const A g = (A)to_f32(in[2 * (int64_t)width + c]);
+    A keep, add;
+    gru_gates<A>((A)to_f32(in[c]) + bias_z, (A)to_f32(in[width + c]) + bias_x, keep, add);
+    s = keep * s + add;
+    out[(int64_t)t * out_stride + c] = from_f32<T>((float)(s * (g * logistic(g))));
+  }
+}
+
+template <typename T>
+static int gated_scan_launch(const void* zxg, int64_t in_stride, const float* bz, const float* bx, float* state,
+                             const int* cu, const int* slots, void* out, int64_t out_stride, int num_requests,
+                             int width, int num_slots, int chunk, int chunks_per_request, float* summaries,
+                             hipStream_t stream) {
+  const int col_blocks = ceil_div(width, 64);
+  if (chunk <= 0) {
+    dim3 grid(col_blocks, num_requests);
+    gated_scan_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, state, cu, slots, (T*)out,
+                                                  out_stride, width, num_slots);
+    MI_CHECK_LAUNCH("gated_scan");
+    return MI_OK;
+  }
+  dim3 grid(col_blocks, chunks_per_request, num_requests);
+  gated_scan_summaries_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, width,
+                                                          chunk, chunks_per_request);
+  MI_CHECK_LAUNCH("gated_scan (summaries)");
+  gated_scan_carry_kernel<<<dim3(col_blocks, num_requests), 64, 0, stream>>>(summaries, state, cu, slots, width, chunk,
+                                                                             chunks_per_request, num_slots);
+  MI_CHECK_LAUNCH("gated_scan (carry)");
+  gated_scan_outputs_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, (T*)out,
+                                                        out_stride, width, chunk, chunks_per_request);
+  MI_CHECK_LAUNCH("gated_scan (outputs)");
+  return MI_OK;
+}
+
+// `chunk` = 0: the sequential form.  `chunk` > 0: the chunked form; no request may bring more
+// than chunk * chunks_per_request rows (the caller's bound), and `summaries` holds
+// num_requests * chunks_per_request * 2 * width floats.
+extern "C" int mi_gated_scan(int dtype, const void* zxg, int64_t in_stride, const float* bz, const float* bx,
+                             float* state, const int* cu, const int* slots, void* out, int64_t out_stride,
+                             int num_requests, int width, int num_slots, int chunk, int chunks_per_request,
+                             float* summaries, hipStream_t stream) {
+  MI_REQUIRE(num_requests >= 0 && width > 0 && num_slots >= 0, "gated_scan: bad sizes requests=%d width=%d slots=%d",
+             num_requests, width, num_slots);
+  MI_REQUIRE(in_stride >= 3 * (int64_t)width && out_stride >= width, "gated_scan: rows hold [z | x | g], %d each", width);
+  MI_REQUIRE(chunk >= 0 && (chunk == 0 || (chunks_per_request > 0 && summaries != nullptr)),
+             "gated_scan: the chunked form needs a chunk count and a summaries buffer");
+  MI_REQUIRE(num_requests <= 65535 && chunks_per_request <= 65535, "gated_scan: too many requests or chunks for one launch");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "gated_scan: unknown dtype %d", dtype);
+  if (num_requests == 0) return MI_OK;
+  if (dtype == MI_F32)
+    return gated_scan_launch<float>(zxg, in_stride, bz, bx, state, cu, slots, out, out_stride, num_requests, width,
+                                    num_slots, chunk, chunks_per_request, summaries, stream);
+  return gated_scan_launch<bf16_t>(zxg, in_stride, bz, bx, state, cu, slots, out, out_stride, num_requests, width,
+                                   num_slots, chunk, chunks_per_request, summaries, stream);
+}
+
+// ---------------------------------------------------------------------------
+// q and k normed over their whole projection, and the cache write.
+//   row layout of qk: [q: q_width | k: kv_heads * head_dim]
+//   q <- q * rsqrt(mean(q^2) + eps) * qw      (in place)
+//   key page slot   <- k * rsqrt(mean(k^2) + eps) * kw
+//   value page slot <- k as it came           (the values are the keys before their norm)
+// Page layouts and slot numbering are those of rope_kv_write.  kv_heads = 0: q only.
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
+    T* __restrict__ qk, int64_t row_stride, const float* __restrict__ qw, const float* __restrict__ kw,
+    const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int q_width,
+    int kv_heads, int head_dim, int page_size, int v_transposed, float eps) {
+  using A = typename Wide<T>::type;
+  __shared__ A scratch[4];
+  const int t = blockIdx.x;
+  T* row = qk + (int64_t)t * row_stride;
+  const int k_width = kv_heads * head_dim;
+  A q_squares = 0, k_squares = 0;
+  for (int i = threadIdx.x; i < q_width; i += blockDim.x) {
+    const A v = (A)to_f32(row[i]);
+    q_squares += v * v;
+  }
+  for (int i = threadIdx.x; i < k_width; i += blockDim.x) {
+    const A v = (A)to_f32(row[q_width + i]);
+    k_squares += v * v;
+  }
+  const A q_inv = inv_root(block_total<A>(q_squares, scratch) / (A)q_width, (A)eps);
+  for (int i = threadIdx.x; i < q_width; i += blockDim.x)
+    row[i] = from_f32<T>((float)(((A)to_f32(row[i]) * q_inv) * (A)qw[i]));
+  if (k_width == 0 || slot_mapping == nullptr) return;
+  const A k_inv = inv_root(block_total<A>(k_squares, scratch) / (A)k_width, (A)eps);
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size;
+  for (int e = threadIdx.x; e < k_width; e += blockDim.x) {
+    const int h = e / head_dim, d = e % head_dim;
+    const T raw = row[q_width + e];
+    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
+    k_pages[chunk + (int64_t)off * head_dim + d] = from_f32<T>((float)(((A)to_f32(raw) * k_inv) * (A)kw[e]));
+    v_pages[v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * head_dim + d] = raw;
+  }
+}
+
+extern "C" int mi_qk_norm_kv_write(int dtype, void* qk, int64_t row_stride, const float* qw, const float* kw,
+                                   const int* slot_mapping, void* k_pages, void* v_pages, int num_tokens, int q_width,
+                                   int kv_heads, int head_dim, int page_size, int num_pages, int v_transposed,
+                                   float eps, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && q_width > 0 && kv_heads >= 0 && head_dim > 0,
+             "qk_norm_kv_write: bad sizes tokens=%d q_width=%d kv_heads=%d head_dim=%d", num_tokens, q_width, kv_heads,
+             head_dim);
+  MI_REQUIRE(row_stride >= (int64_t)q_width + (int64_t)kv_heads * head_dim,
+             "qk_norm_kv_write: row stride %lld is shorter than q and k together", (long long)row_stride);
+  MI_REQUIRE(kv_heads == 0 || slot_mapping == nullptr || (page_size > 0 && num_pages > 0 && k_pages && v_pages && kw),
+             "qk_norm_kv_write: pages and the key norm's weight are needed to write keys and values");
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "qk_norm_kv_write: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    qk_norm_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)qk, row_stride, qw, kw, slot_mapping,
+                                                                   (float*)k_pages, (float*)v_pages, q_width, kv_heads,
+                                                                   head_dim, page_size, v_transposed, eps);
+  } else {
+    qk_norm_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)qk, row_stride, qw, kw, slot_mapping,
+                                                                    (bf16_t*)k_pages, (bf16_t*)v_pages, q_width,
+                                                                    kv_heads, head_dim, page_size, v_transposed, eps);
+  }
+  MI_CHECK_LAUNCH("qk_norm_kv_write");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// PolyNorm over a token's feed-forward values z [width]:
+//   out = a * z / rms(z) + b * z^2 / rms(z^2) + c * z^3 / rms(z^3) + e,   rms(v) = sqrt(mean(v^2) + eps)
+// `coef` = (a, b, c, e) float32.  One block a row.
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void poly_norm_kernel(const T* __restrict__ z, int64_t in_stride,
+                                                        const float* __restrict__ coef, T* __restrict__ out,
+                                                        int64_t out_stride, int width, float eps) {
+  using A = typename Wide<T>::type;
+  __shared__ A scratch[4];
+  const int t = blockIdx.x;
+  const T* row = z + (int64_t)t * in_stride;
+  A s2 = 0, s4 = 0, s6 = 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const A v = (A)to_f32(row[i]);
+    const A v2 = v * v;
+    s2 += v2;
+    s4 += v2 * v2;
+    s6 += v2 * v2 * v2;
+  }
+  const A n = (A)width;
+  const A i1 = inv_root(block_total<A>(s2, scratch) / n, (A)eps);
+  const A i2 = inv_root(block_total<A>(s4, scratch) / n, (A)eps);
+  const A i3 = inv_root(block_total<A>(s6, scratch) / n, (A)eps);
+  const A a = (A)coef[0] * i1, b = (A)coef[1] * i2, c = (A)coef[2] * i3, e = (A)coef[3];
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const A v = (A)to_f32(row[i]);
+    const A v2 = v * v;
+    out[(int64_t)t * out_stride + i] = from_f32<T>((float)(a * v + b * v2 + c * (v2 * v) + e));
+  }
+}
+
+extern "C" int mi_poly_norm(int dtype, const void* z, int64_t in_stride, const float* coef, void* out,
+                            int64_t out_stride, int num_tokens, int width, float eps, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && width > 0 && in_stride >= width && out_stride >= width,
+             "poly_norm: bad sizes tokens=%d width=%d", num_tokens, width);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "poly_norm: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32) {
+    poly_norm_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)z, in_stride, coef, (float*)out, out_stride,
+                                                            width, eps);
+  } else {
+    poly_norm_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)z, in_stride, coef, (bf16_t*)out,
+                                                             out_stride, width, eps);
+  }
+  MI_CHECK_LAUNCH("poly_norm");
+  return MI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// out[t, j] = gelu_tanh(gate[t, j]) * table[ids[t], first_col + j],  j < width
+//   gelu_tanh(z) = z/2 * (1 + tanh(sqrt(2/pi) * (z + 0.044715 z^3)))
+// ---------------------------------------------------------------------------
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_table_rows_kernel(
+    const T* __restrict__ gate, int64_t gate_stride, const T* __restrict__ table, int64_t table_stride,
+    const int* __restrict__ ids, T* __restrict__ out, int width, int first_col, int64_t total) {
+  using A = typename Wide<T>::type;
+  const int64_t at = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (at >= total) return;
+  const int64_t t = at / width;
+  const int j = (int)(at % width);
+  const A z = (A)to_f32(gate[t * gate_stride + j]);
+  const A inner = (A)0.7978845608028654 * (z + (A)0.044715 * z * z * z);
+  const A act = (A)0.5 * z * ((A)1 + tanh_of(inner));
+  const A e = (A)to_f32(table[(int64_t)ids[t] * table_stride + first_col + j]);
+  out[at] = from_f32<T>((float)(act * e));
+}
+
+extern "C" int mi_gated_table_rows(int dtype, const void* gate, int64_t gate_stride, const void* table,
+                                   int64_t table_stride, const int* ids, void* out, int num_tokens, int width,
+                                   int first_col, int vocab, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && width > 0 && first_col >= 0 && vocab > 0 && gate_stride >= width &&
+                 table_stride >= (int64_t)first_col + width,
+             "gated_table_rows: bad sizes tokens=%d width=%d first_col=%d", num_tokens, width, first_col);
+  MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "gated_table_rows: unknown dtype %d", dtype);
+  if (num_tokens == 0) return MI_OK;
+  const int64_t total = (int64_t)num_tokens * width;
+  const unsigned blocks = (unsigned)ceil_div64(total, 256);
+  if (dtype == MI_F32) {
+    gated_table_rows_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate, gate_stride, (const float*)table,
+                                                               table_stride, ids, (float*)out, width, first_col, total);
+  } else {
+    gated_table_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gate, gate_stride, (const bf16_t*)table,
+                                                                table_stride, ids, (bf16_t*)out, width, first_col, total);
+  }
+  MI_CHECK_LAUNCH("gated_table_rows");
+  return MI_OK;
+}

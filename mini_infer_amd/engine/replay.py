@@ -35,7 +35,7 @@ def build_parser() -> argparse.ArgumentParser:
         help="most tokens live requests hold at any time (each rounded up to a multiple of 64)",
     )
     parser.add_argument("--block-size", type=int, default=DEFAULT_REPLAY_BLOCK_SIZE)
-    parser.add_argument("--max-concurrent", type=int, default=64)
+    parser.add_argument("--max-concurrent", type=int, default=4, help="state slots: the most requests live at a time")
     parser.add_argument("--device", default="cuda:0")
     return parser
 

@@ -1078,6 +1078,211 @@ def paged_attention(
     return out
 
 
+# ----------------------------------------------------------------------------
+# sublayers that add their own normed output to the stream, and what goes with them
+# ----------------------------------------------------------------------------
+
+
+def _need_f32(name: str, t: torch.Tensor | None) -> None:
+    if t is not None and t.dtype != torch.float32:
+        raise KernelShapeError(f"{name} stays float32, got {t.dtype}")
+
+
+def embed_sinusoid(
+    table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor, scale: float,
+    want_cast: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """`float32(table[ids]) * scale + wave(positions)`: column 2i of the wave is sin(p * freq[i]),
+    column 2i+1 the cosine.  `freq` is float64 [ceil(H/2)].  Returns the float32 stream [T, H] and,
+    with `want_cast`, the same rows in the table's dtype."""
+    _need_cuda(table, ids, positions, freq)
+    for name, t in (("table", table), ("ids", ids), ("positions", positions), ("freq", freq)):
+        _need_contiguous(name, t)
+    _need_int32("ids", ids)
+    _need_int32("positions", positions)
+    vocab, hidden = table.shape
+    if freq.dtype != torch.float64 or freq.numel() != (hidden + 1) // 2:
+        raise KernelShapeError(f"freq must be float64 [{(hidden + 1) // 2}], got {freq.dtype} x {freq.numel()}")
+    if positions.numel() != ids.numel():
+        raise KernelShapeError("embed_sinusoid: one position per token id")
+    out = torch.empty((ids.numel(), hidden), dtype=torch.float32, device=table.device)
+    cast = torch.empty((ids.numel(), hidden), dtype=table.dtype, device=table.device) if want_cast else None
+    library.check(
+        library.load().mi_embed_sinusoid(
+            _dtype_code(table), _ptr(table), _ptr(ids), _ptr(positions), _ptr(freq), _ptr(out), _ptr(cast),
+            ids.numel(), hidden, vocab, float(scale), _stream(),
+        )
+    )
+    return out, cast
+
+
+def norm_scale_add(
+    y: torch.Tensor, residual: torch.Tensor, gain: torch.Tensor | None, scale: torch.Tensor | None, eps: float,
+    want_cast: bool = False,
+) -> torch.Tensor | None:
+    """`residual += y * rsqrt(mean(y^2) + eps) * gain * scale` row by row, in place (float32).
+    `gain`: one float32 number or None; `scale`: float32 [H] or None.  With `want_cast` the new
+    rows are returned in the dtype of `y` as well."""
+    _need_cuda(y, residual, gain, scale)
+    _need_contiguous("residual", residual)
+    _need_contiguous("scale", scale)
+    _need_f32("residual", residual)
+    _need_f32("gain", gain)
+    _need_f32("scale", scale)
+    if y.dim() != 2 or y.stride(1) != 1 or tuple(y.shape) != tuple(residual.shape):
+        raise KernelShapeError(f"norm_scale_add: y {tuple(y.shape)} does not fit the stream {tuple(residual.shape)}")
+    tokens, hidden = residual.shape
+    if gain is not None and gain.numel() != 1:
+        raise KernelShapeError(f"norm_scale_add: the gain is one number, got {gain.numel()}")
+    if scale is not None and scale.numel() != hidden:
+        raise KernelShapeError(f"norm_scale_add: the scale has {scale.numel()} entries for {hidden} columns")
+    cast = torch.empty((tokens, hidden), dtype=y.dtype, device=y.device) if want_cast else None
+    library.check(
+        library.load().mi_norm_scale_add(
+            _dtype_code(y), _ptr(y), y.stride(0), _ptr(residual), _ptr(gain), _ptr(scale), _ptr(cast), tokens, hidden,
+            float(eps), _stream(),
+        )
+    )
+    return cast
+
+
+def cast_rows(residual: torch.Tensor) -> torch.Tensor:
+    """The float32 stream rounded to bfloat16."""
+    _need_cuda(residual)
+    _need_contiguous("residual", residual)
+    _need_f32("residual", residual)
+    out = torch.empty(residual.shape, dtype=torch.bfloat16, device=residual.device)
+    library.check(library.load().mi_cast_rows(_ptr(residual), _ptr(out), residual.numel(), _stream()))
+    return out
+
+
+GATED_SCAN_CHUNK = 64  # rows of a chunk of the chunked recurrence
+GATED_SCAN_SEQUENTIAL_ROWS = 128  # portions up to this many rows are walked by one thread a column
+
+
+def gated_scan(
+    zxg: torch.Tensor, bias_z: torch.Tensor, bias_x: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
+    slots: torch.Tensor, max_rows: int | None,
+) -> torch.Tensor:
+    """minGRU over the rows of a step.  `zxg` [T, 3W] holds the projections [z | x | g] of every
+    token; request b owns rows `cu_seqlens[b]..cu_seqlens[b+1]` and the state row `state[slots[b]]`
+    (float32 [slots + 1, W]; a negative slot means the last row, which is nobody's).  Returns
+    `S_t * silu(g_t)` [T, W]; the state rows are advanced in place.  `max_rows`: the most rows a
+    request brings, if the host knows (long portions then run chunk by chunk in parallel)."""
+    _need_cuda(zxg, bias_z, bias_x, state, cu_seqlens, slots)
+    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("state", state), ("cu_seqlens", cu_seqlens), ("slots", slots)):
+        _need_contiguous(name, t)
+    _need_int32("cu_seqlens", cu_seqlens)
+    _need_int32("slots", slots)
+    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("state", state)):
+        _need_f32(name, t)
+    if zxg.dim() != 2 or zxg.stride(1) != 1 or zxg.shape[1] % 3 != 0:
+        raise KernelShapeError(f"gated_scan: rows hold [z | x | g], got {tuple(zxg.shape)} strides {zxg.stride()}")
+    tokens, width = zxg.shape[0], zxg.shape[1] // 3
+    requests = slots.numel()
+    if cu_seqlens.numel() != requests + 1 or bias_z.numel() != width or bias_x.numel() != width:
+        raise KernelShapeError("gated_scan: one more boundary than requests, one bias per column")
+    if state.dim() != 2 or state.shape[1] != width or state.shape[0] < 2:
+        raise KernelShapeError(f"gated_scan: state is [slots + 1, {width}], got {tuple(state.shape)}")
+    out = torch.empty((tokens, width), dtype=zxg.dtype, device=zxg.device)
+    chunk = chunks = 0
+    summaries = None
+    if max_rows is not None and max_rows > GATED_SCAN_SEQUENTIAL_ROWS:
+        chunk, chunks = GATED_SCAN_CHUNK, -(-max_rows // GATED_SCAN_CHUNK)
+        summaries = torch.empty((requests, chunks, 2, width), dtype=torch.float32, device=zxg.device)
+    library.check(
+        library.load().mi_gated_scan(
+            _dtype_code(zxg), _ptr(zxg), zxg.stride(0), _ptr(bias_z), _ptr(bias_x), _ptr(state), _ptr(cu_seqlens),
+            _ptr(slots), _ptr(out), out.stride(0), requests, width, state.shape[0] - 1, chunk, chunks, _ptr(summaries),
+            _stream(),
+        )
+    )
+    return out
+
+
+def qk_norm_kv_write(
+    qk: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor | None, slot_mapping: torch.Tensor | None,
+    k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, *, q_width: int, kv_heads: int, head_dim: int,
+    eps: float, v_transposed: bool = False,
+) -> None:
+    """`qk` [T, q_width + kv_heads*head_dim]: q is normed in place over its whole width
+    (`q * rsqrt(mean(q^2) + eps) * q_weight`); k, normed the same way with `k_weight`, goes to its
+    key-page slot and k as it came to the value-page slot.  `kv_heads=0`: q only."""
+    _need_cuda(qk, q_weight, k_weight, slot_mapping, k_pages, v_pages)
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight), ("slot_mapping", slot_mapping),
+                    ("k_pages", k_pages), ("v_pages", v_pages)):
+        _need_contiguous(name, t)
+    _need_int32("slot_mapping", slot_mapping)
+    _need_f32("q_weight", q_weight)
+    _need_f32("k_weight", k_weight)
+    if qk.dim() != 2 or qk.stride(1) != 1 or qk.shape[1] < q_width + kv_heads * head_dim:
+        raise KernelShapeError(f"qk_norm_kv_write: rows hold q and k, got {tuple(qk.shape)} strides {qk.stride()}")
+    if q_weight.numel() != q_width or (kv_heads > 0 and (k_weight is None or k_weight.numel() != kv_heads * head_dim)):
+        raise KernelShapeError("qk_norm_kv_write: one norm weight per column of q and of k")
+    tokens = qk.shape[0]
+    page_size = num_pages = 0
+    if kv_heads > 0:
+        if slot_mapping is None or k_pages is None or v_pages is None:
+            raise KernelShapeError("writing keys and values needs slot_mapping, k_pages and v_pages")
+        if k_pages.dtype != qk.dtype or v_pages.dtype != qk.dtype:
+            raise KernelShapeError(f"pages are {k_pages.dtype}, activations {qk.dtype}")
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+            raise KernelShapeError(f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}")
+        _check_v_pages(k_pages, v_pages, v_transposed)
+        if slot_mapping.numel() != tokens:
+            raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    library.check(
+        library.load().mi_qk_norm_kv_write(
+            _dtype_code(qk), _ptr(qk), qk.stride(0), _ptr(q_weight), _ptr(k_weight),
+            _ptr(slot_mapping) if kv_heads > 0 else None, _ptr(k_pages) if kv_heads > 0 else None,
+            _ptr(v_pages) if kv_heads > 0 else None, tokens, q_width, kv_heads, head_dim, page_size, num_pages,
+            int(v_transposed), float(eps), _stream(),
+        )
+    )
+
+
+def poly_norm(z: torch.Tensor, coefficients: torch.Tensor, eps: float) -> torch.Tensor:
+    """`a N(z) + b N(z^2) + c N(z^3) + e` row by row, N(v) = v / sqrt(mean(v^2) + eps);
+    `coefficients` = (a, b, c, e) float32."""
+    _need_cuda(z, coefficients)
+    _need_contiguous("coefficients", coefficients)
+    _need_f32("coefficients", coefficients)
+    if z.dim() != 2 or z.stride(1) != 1 or coefficients.numel() != 4:
+        raise KernelShapeError(f"poly_norm: z is [T, width], four coefficients; got {tuple(z.shape)}, {coefficients.numel()}")
+    out = torch.empty(z.shape, dtype=z.dtype, device=z.device)
+    library.check(
+        library.load().mi_poly_norm(
+            _dtype_code(z), _ptr(z), z.stride(0), _ptr(coefficients), _ptr(out), out.stride(0), z.shape[0], z.shape[1],
+            float(eps), _stream(),
+        )
+    )
+    return out
+
+
+def gated_table_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, first_col: int) -> torch.Tensor:
+    """`gelu_tanh(gate) * table[ids, first_col : first_col + width]` for `gate` [T, width]."""
+    _need_cuda(gate, table, ids)
+    _need_contiguous("table", table)
+    _need_contiguous("ids", ids)
+    _need_int32("ids", ids)
+    if gate.dim() != 2 or gate.stride(1) != 1 or table.dim() != 2 or table.dtype != gate.dtype:
+        raise KernelShapeError("gated_table_rows: gate is [T, width], the table [vocab, columns] of the same dtype")
+    tokens, width = gate.shape
+    if ids.numel() != tokens or first_col < 0 or first_col + width > table.shape[1]:
+        raise KernelShapeError(
+            f"gated_table_rows: columns {first_col}..{first_col + width} of a table with {table.shape[1]}, {ids.numel()} ids for {tokens} rows"
+        )
+    out = torch.empty((tokens, width), dtype=gate.dtype, device=gate.device)
+    library.check(
+        library.load().mi_gated_table_rows(
+            _dtype_code(gate), _ptr(gate), gate.stride(0), _ptr(table), table.stride(0), _ptr(ids), _ptr(out), tokens,
+            width, int(first_col), table.shape[0], _stream(),
+        )
+    )
+    return out
+
+
 def sample(
     logits: torch.Tensor,
     temperature: torch.Tensor,

@@ -46,6 +46,8 @@ class GQAttention(Mixer):
         *,
         window: int | None = None,
         scale: float | None = None,
+        names: tuple[str, str, str, str] = ("q_proj", "k_proj", "v_proj", "o_proj"),
+        suffix: str = ".weight",
     ) -> None:
         super().__init__(dtype, device)
         if num_heads % num_kv_heads != 0:
@@ -71,8 +73,12 @@ class GQAttention(Mixer):
         ):
             raise ValueError(f"score slopes must be float32 [{num_heads}], got {self.slopes.dtype} {tuple(self.slopes.shape)}")
         q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim
-        self.qkv = Linear(hidden_size, [q_width, kv_width, kv_width], ["q_proj", "k_proj", "v_proj"], dtype, device)
-        self.out = Linear(q_width, hidden_size, "o_proj", dtype, device)
+        self.qkv = self._input_projection(hidden_size, q_width, kv_width, names, suffix)
+        self.out = Linear(q_width, hidden_size, names[3], dtype, device, suffix=suffix)
+
+    def _input_projection(self, hidden_size: int, q_width: int, kv_width: int, names, suffix: str) -> Linear:
+        """The stacked product that feeds the attention: q | k | v here."""
+        return Linear(hidden_size, [q_width, kv_width, kv_width], list(names[:3]), self.dtype, self.device, suffix=suffix)
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
         return {**self.qkv.param_specs(prefix), **self.out.param_specs(prefix)}
@@ -167,6 +173,79 @@ class GQAttention(Mixer):
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few, slopes=self.slopes,
         )
+
+
+class KeysAsValuesAttention(GQAttention):
+    """Grouped-query attention without a value projection: the values are the keys as
+    projected, before the keys' norm.  Queries and keys are RMS-normed over their WHOLE
+    projection (all heads at once, one weight per column) before they are split into heads.
+    Positions enter the scores only if a position encoding is given (none: the window and the
+    causal order are all the layer knows of positions).
+
+    The pages hold two streams as everywhere else: normed keys in the key pages, the un-normed
+    key projection in the value pages, so the paged attention kernels run unchanged."""
+
+    can_defer_output = False
+    takes_scaled_rows = False
+
+    def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, dtype, device, *, norm_eps: float,
+                 window=None, scale=None, names=("q", "k", "", "o"), suffix="",
+                 norm_names=("q.norm", "k.norm")) -> None:
+        super().__init__(hidden_size, num_heads, num_kv_heads, head_dim, None, dtype, device, window=window,
+                         scale=scale, names=names, suffix=suffix)
+        self.norm_eps = float(norm_eps)
+        self.norm_names = tuple(norm_names)
+        self.q_norm: torch.Tensor | None = None
+        self.k_norm: torch.Tensor | None = None
+
+    def _input_projection(self, hidden_size, q_width, kv_width, names, suffix):
+        return Linear(hidden_size, [q_width, kv_width], [names[0], names[1]], self.dtype, self.device, suffix=suffix)
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        q_width, kv_width = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        return {
+            **super().param_specs(prefix),
+            prefix + self.norm_names[0]: ParamSpec((q_width,), init="norm_weight", dtype="float32"),
+            prefix + self.norm_names[1]: ParamSpec((kv_width,), init="norm_weight", dtype="float32"),
+        }
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        super().load_params(prefix, get)
+        self.q_norm = get(prefix + self.norm_names[0]).float().contiguous()
+        self.k_norm = get(prefix + self.norm_names[1]).float().contiguous()
+
+    def wants_scaled_rows(self, rows: int) -> bool:
+        return False
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        assert cache.group is not None and cache.k_pages is not None and cache.v_pages is not None
+        assert self.qkv.weight is not None and self.q_norm is not None, "attention used before its weights were loaded"
+        if isinstance(x, ops.ScaledRows):
+            x = x.finish()
+        q_width = self.num_heads * self.head_dim
+        if writes_cache:
+            qk = self.qkv.forward(x)
+            kv_heads, slots = self.num_kv_heads, ctx.slot_mapping[cache.group]
+        else:
+            qk = ops.linear(x, self.qkv.weight[:q_width])
+            kv_heads, slots = 0, None
+        ops.qk_norm_kv_write(
+            qk, self.q_norm, self.k_norm if writes_cache else None, slots, cache.k_pages, cache.v_pages,
+            q_width=q_width, kv_heads=kv_heads, head_dim=self.head_dim, eps=self.norm_eps,
+            v_transposed=cache.v_transposed,
+        )
+        return self._project(self._attend(qk, ctx, cache))
+
+
+@register_mixer("keys_as_values_attention")
+def build_keys_as_values_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> KeysAsValuesAttention:
+    extra = {k: desc[k] for k in ("names", "suffix", "norm_names") if k in desc}
+    if "names" in extra:
+        extra["names"] = tuple(extra["names"])
+    return KeysAsValuesAttention(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["num_kv_heads"]), int(desc["head_dim"]), dtype, device,
+        norm_eps=float(desc["norm_eps"]), window=desc.get("window"), scale=desc.get("scale"), **extra,
+    )
 
 
 @register_mixer("gqa_attention")

@@ -206,6 +206,18 @@ class Norm(Part):
     ) -> torch.Tensor:
         raise NotImplementedError
 
+    def add_output(
+        self,
+        y: torch.Tensor,
+        residual: torch.Tensor,
+        scale: torch.Tensor | None = None,
+        want_cast: bool = False,
+    ) -> torch.Tensor | None:
+        """The other place a norm can stand: on a sublayer's OUTPUT.  `residual += norm(y) * scale`
+        in place (float32; `scale` float32 [hidden] or None); with `want_cast` the new rows are
+        returned in the compute dtype too.  Only norms that a block uses this way implement it."""
+        raise NotImplementedError(f"{type(self).__name__} cannot stand on a sublayer's output")
+
 
 @dataclasses.dataclass
 class RotaryTables:

@@ -121,3 +121,98 @@ def build_pre_norm_block(desc: dict, dtype: torch.dtype, device, shared: dict | 
         dtype,
         device,
     )
+
+
+class OutputNormBlock(Block):
+    """Sublayers that read the stream itself and are normed on the way OUT:
+
+        x <- x + scale1 * norm1(mixer(x))
+        x <- x + scale2 * norm2(feed_forward(x))        (a layer may have none)
+        x <- x + side_norm(side(x, tokens))             (a layer may have none)
+
+    `scale1`, `scale2` are per-column layer scales (float32).  Every add is done here, by the
+    norm's kernel, so the block hands nothing pending to what follows.  In the bfloat16 engine
+    the same kernel leaves the stream's copy in bfloat16 for the next sublayer's products."""
+
+    takes_pending_products = False
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, feed_forward: FeedForward | None,
+                 side: FeedForward | None, side_norm: Norm | None, hidden_size: int, layer_scale: bool,
+                 names: dict[str, str], dtype: torch.dtype, device) -> None:
+        super().__init__(dtype, device)
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.ffn_norm, self.feed_forward = ffn_norm, feed_forward
+        self.side, self.side_norm = side, side_norm
+        self.hidden_size, self.layer_scale, self.names = hidden_size, layer_scale, names
+        self.mixer_scale: torch.Tensor | None = None
+        self.ffn_scale: torch.Tensor | None = None
+
+    def _children(self):
+        parts = [(self.names["mixer_norm"], self.mixer_norm), (self.names["mixer"], self.mixer)]
+        if self.feed_forward is not None:
+            parts += [(self.names["ffn_norm"], self.ffn_norm), (self.names["feed_forward"], self.feed_forward)]
+        if self.side is not None:
+            parts += [(self.names["side"], self.side), (self.names["side_norm"], self.side_norm)]
+        return parts
+
+    @property
+    def graph_safe(self) -> bool:  # type: ignore[override]
+        return all(part.graph_safe for _, part in self._children())
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        specs: dict[str, ParamSpec] = {}
+        for sub, part in self._children():
+            specs.update(part.param_specs(prefix + sub))
+        if self.layer_scale:
+            specs[prefix + self.names["mixer_scale"]] = ParamSpec((self.hidden_size,), init="norm_weight", dtype="float32")
+            if self.feed_forward is not None:
+                specs[prefix + self.names["ffn_scale"]] = ParamSpec((self.hidden_size,), init="norm_weight", dtype="float32")
+        return specs
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        for sub, part in self._children():
+            part.load_params(prefix + sub, get)
+        if self.layer_scale:
+            self.mixer_scale = get(prefix + self.names["mixer_scale"]).float().contiguous()
+            if self.feed_forward is not None:
+                self.ffn_scale = get(prefix + self.names["ffn_scale"]).float().contiguous()
+
+    def forward(self, delta, residual: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        from mini_infer_amd.parts.embedding import STREAM_CAST, stream_for_products
+
+        if delta is not None:  # a block of another arrangement left its output to be added
+            residual.add_(delta.finish() if hasattr(delta, "finish") else delta)
+        narrow = self.dtype != torch.float32
+
+        def added(cast):
+            if cast is not None:
+                ctx.shared[STREAM_CAST] = (residual, cast)
+
+        mixed = self.mixer.forward(stream_for_products(residual, ctx, self.dtype), ctx, cache, writes_cache)
+        added(self.mixer_norm.add_output(mixed, residual, self.mixer_scale, narrow))
+        if self.feed_forward is not None:
+            fed = self.feed_forward.forward(stream_for_products(residual, ctx, self.dtype), ctx)
+            added(self.ffn_norm.add_output(fed, residual, self.ffn_scale, narrow))
+        if self.side is not None:
+            extra = self.side.forward(stream_for_products(residual, ctx, self.dtype), ctx)
+            added(self.side_norm.add_output(extra, residual, None, narrow))
+        return None
+
+
+@register_block("output_norm")
+def build_output_norm_block(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> OutputNormBlock:
+    """`desc`: `norm` (for both sublayers), `mixer`, optional `feed_forward`, optional `side` with
+    `side_norm`, `hidden_size`, `layer_scale` (whether the layer has per-column scales) and
+    `names` (each part's name inside the layer)."""
+    shared = {} if shared is None else shared
+
+    def build(registry, part):
+        return registry.lookup(part["kind"])(part, dtype, device, shared) if part is not None else None
+
+    ffn, side = desc.get("feed_forward"), desc.get("side")
+    return OutputNormBlock(
+        build(NORMS, desc["norm"]), build(MIXERS, desc["mixer"]),
+        build(NORMS, desc["norm"]) if ffn is not None else None, build(FEED_FORWARDS, ffn),
+        build(FEED_FORWARDS, side), build(NORMS, desc.get("side_norm")) if side is not None else None,
+        int(desc["hidden_size"]), bool(desc.get("layer_scale", False)), dict(desc["names"]), dtype, device,
+    )

@@ -40,6 +40,49 @@ class TokenEmbedding(Embedding):
         return ops.embed_gather(self.weight, ctx.token_ids)
 
 
+SINUSOID_BASE = 10000.0
+STREAM_CAST = "stream_cast"  # key in `StepContext.shared`: (the stream, its latest copy in the compute dtype)
+
+
+def stream_for_products(residual: torch.Tensor, ctx: StepContext, dtype: torch.dtype) -> torch.Tensor:
+    """The float32 stream as the products of a sublayer that reads it un-normed take it: itself
+    in the 32-bit engine, else its copy in the compute dtype (left in `ctx.shared` by whichever
+    kernel last wrote the stream, or made here)."""
+    if dtype == torch.float32:
+        return residual
+    kept = ctx.shared.get(STREAM_CAST)
+    if kept is not None and kept[0] is residual:
+        return kept[1]
+    cast = ops.cast_rows(residual)
+    ctx.shared[STREAM_CAST] = (residual, cast)
+    return cast
+
+
+class ScaledSinusoidEmbedding(TokenEmbedding):
+    """`table[token] * scale` plus a fixed wave of the position: column 2i gets
+    sin(p * base^(-2i/H)), column 2i+1 the cosine of the same angle.  Frequencies are made in
+    64-bit on the host; the kernel takes the angle in float32 (64-bit in the 32-bit engine)."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float, dtype: torch.dtype, device,
+                 base: float = SINUSOID_BASE) -> None:
+        super().__init__(vocab_size, hidden_size, name, dtype, device)
+        self.scale = float(scale)
+        pairs = torch.arange((hidden_size + 1) // 2, dtype=torch.float64)
+        self.freq_host = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * pairs / hidden_size)
+        self._freq: torch.Tensor | None = None
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        assert self.weight is not None, "embedding used before its table was loaded"
+        if self._freq is None:
+            self._freq = self.freq_host.to(self.device).contiguous()
+        residual, cast = ops.embed_sinusoid(
+            self.weight, ctx.token_ids, ctx.positions, self._freq, self.scale, want_cast=self.dtype != torch.float32
+        )
+        if cast is not None:
+            ctx.shared[STREAM_CAST] = (residual, cast)
+        return residual
+
+
 class OutputHead(Head):
     graph_safe = True
 
@@ -87,6 +130,14 @@ class OutputHead(Head):
 @register_embedding("token_embedding")
 def build_token_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> TokenEmbedding:
     return TokenEmbedding(int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), dtype, device)
+
+
+@register_embedding("scaled_sinusoid_embedding")
+def build_scaled_sinusoid_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ScaledSinusoidEmbedding:
+    return ScaledSinusoidEmbedding(
+        int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), float(desc["scale"]), dtype, device,
+        base=float(desc.get("base", SINUSOID_BASE)),
+    )
 
 
 @register_head("linear_head")

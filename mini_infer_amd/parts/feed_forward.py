@@ -63,3 +63,115 @@ def build_swiglu(desc: dict, dtype: torch.dtype, device, shared: dict | None = N
     if activation != "silu":
         raise NotImplementedError(f"gated feed-forward activation {activation!r}; only 'silu' is built")
     return SwiGLU(int(desc["hidden_size"]), int(desc["intermediate_size"]), dtype, device)
+
+
+class PolyNormFeedForward(FeedForward):
+    """Dense, ungated: `down(act(up(x)))` with a polynomial activation of normed powers,
+
+        act(z) = a N(z) + b N(z^2) + c N(z^3) + e,     N(v) = v / sqrt(mean(v^2) + eps)
+
+    where the powers are elementwise and the mean runs over a token's feed-forward values.
+    The four numbers are one float32 tensor."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, eps: float, dtype: torch.dtype, device, *,
+                 names: tuple[str, str, str] = ("up", "down", "act"), suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.eps = float(eps)
+        self.act_name = names[2]
+        self.up = Linear(hidden_size, intermediate_size, names[0], dtype, device, suffix=suffix)
+        self.down = Linear(intermediate_size, hidden_size, names[1], dtype, device, suffix=suffix)
+        self.coefficients: torch.Tensor | None = None
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {**self.up.param_specs(prefix), **self.down.param_specs(prefix),
+                prefix + self.act_name: ParamSpec((4,), dtype="float32")}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.up.load_params(prefix, get)
+        self.down.load_params(prefix, get)
+        self.coefficients = get(prefix + self.act_name).float().contiguous()
+
+    def forward(self, x, ctx: StepContext) -> torch.Tensor:
+        assert self.coefficients is not None, "feed-forward used before its weights were loaded"
+        if isinstance(x, ops.ScaledRows):
+            x = x.finish()
+        return self.down.forward(ops.poly_norm(self.up.forward(x), self.coefficients, self.eps))
+
+
+@register_feed_forward("dense_poly_norm")
+def build_poly_norm_feed_forward(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> PolyNormFeedForward:
+    extra = {k: desc[k] for k in ("names", "suffix") if k in desc}
+    if "names" in extra:
+        extra["names"] = tuple(extra["names"])
+    return PolyNormFeedForward(int(desc["hidden_size"]), int(desc["intermediate_size"]), float(desc["eps"]), dtype, device, **extra)
+
+
+class _SharedTable:
+    """A table that several parts of one model read slices of: loaded once per load pass."""
+
+    def __init__(self, name: str, shape: tuple[int, int]) -> None:
+        self.name, self.shape = name, shape
+        self.tensor: torch.Tensor | None = None
+        self._loaded_with = None
+
+    def load(self, get: TensorGetter) -> torch.Tensor:
+        if self.tensor is None or self._loaded_with is not get:
+            self.tensor, self._loaded_with = get(self.name).contiguous(), get
+        return self.tensor
+
+
+class TokenSideInput(FeedForward):
+    """A per-layer input that depends on the token's identity: the layer's slice
+    `table[token, first : first + dim]` of a table shared by all layers, gated by the stream,
+
+        y = proj(gelu_tanh(gate(x)) * slice)
+
+    `table_name` is the tensor's whole name (it belongs to the model, not to the layer); the
+    parts of one model that name the same table share one copy through `shared`."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, dim: int, first_col: int, table: _SharedTable, dtype: torch.dtype, device, *,
+                 names: tuple[str, str] = ("gate", "proj"), suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        if first_col < 0 or first_col + dim > table.shape[1]:
+            raise ValueError(f"columns {first_col}..{first_col + dim} lie outside a table of {table.shape[1]} columns")
+        self.hidden_size, self.dim, self.first_col, self.table = hidden_size, dim, first_col, table
+        self.gate = Linear(hidden_size, dim, names[0], dtype, device, suffix=suffix)
+        self.proj = Linear(dim, hidden_size, names[1], dtype, device, suffix=suffix)
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {**self.gate.param_specs(prefix), **self.proj.param_specs(prefix),
+                self.table.name: ParamSpec(self.table.shape)}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.gate.load_params(prefix, get)
+        self.proj.load_params(prefix, get)
+        self.table.load(get)
+
+    def forward(self, x, ctx: StepContext) -> torch.Tensor:
+        assert self.table.tensor is not None, "side input used before its table was loaded"
+        if isinstance(x, ops.ScaledRows):
+            x = x.finish()
+        gated = ops.gated_table_rows(self.gate.forward(x), self.table.tensor, ctx.token_ids, self.first_col)
+        return self.proj.forward(gated)
+
+
+@register_feed_forward("token_side_input")
+def build_token_side_input(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> TokenSideInput:
+    shared = {} if shared is None else shared
+    name, shape = str(desc["table_name"]), (int(desc["vocab_size"]), int(desc["table_columns"]))
+    key = ("shared_table", name)
+    table = shared.get(key)
+    if table is None:
+        table = shared[key] = _SharedTable(name, shape)
+    elif table.shape != shape:
+        raise ValueError(f"table {name!r} is described as {shape} and as {table.shape}")
+    extra = {k: desc[k] for k in ("names", "suffix") if k in desc}
+    if "names" in extra:
+        extra["names"] = tuple(extra["names"])
+    return TokenSideInput(int(desc["hidden_size"]), int(desc["dim"]), int(desc["first_col"]), table, dtype, device, **extra)

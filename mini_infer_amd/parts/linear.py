@@ -25,8 +25,11 @@ class Linear(Part):
         names: list[str] | str,
         dtype: torch.dtype,
         device,
+        *,
+        suffix: str = ".weight",
     ) -> None:
         super().__init__(dtype, device)
+        self.suffix = suffix  # what follows a block's name in the checkpoint ("" where the name is the tensor's)
         self.in_features = in_features
         self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
         self.names = [names] if isinstance(names, str) else list(names)
@@ -37,12 +40,12 @@ class Linear(Part):
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
         return {
-            prefix + name + ".weight": ParamSpec((rows, self.in_features))
+            prefix + name + self.suffix: ParamSpec((rows, self.in_features))
             for name, rows in zip(self.names, self.out_splits)
         }
 
     def load_params(self, prefix: str, get: TensorGetter) -> None:
-        blocks = [get(prefix + name + ".weight") for name in self.names]
+        blocks = [get(prefix + name + self.suffix) for name in self.names]
         self.weight = (blocks[0] if len(blocks) == 1 else torch.cat(blocks, dim=0)).contiguous()
 
     def forward(self, x: torch.Tensor, partial_ok: bool = False):

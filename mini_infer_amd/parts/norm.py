@@ -20,17 +20,28 @@ class RMSNorm(Norm):
     takes_partial_sums = True
     takes_pending_products = True
 
-    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device) -> None:
+    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device, name: str = "weight") -> None:
         super().__init__(dtype, device)
         self.hidden_size = hidden_size
         self.eps = float(eps)
+        self.name = name  # the tensor is `prefix + name`
         self.weight: torch.Tensor | None = None
+        self._weight_f32: torch.Tensor | None = None
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
-        return {prefix + "weight": ParamSpec((self.hidden_size,), init="norm_weight")}
+        return {prefix + self.name: ParamSpec((self.hidden_size,), init="norm_weight")}
 
     def load_params(self, prefix: str, get: TensorGetter) -> None:
-        self.weight = get(prefix + "weight").contiguous()
+        self.weight = get(prefix + self.name).contiguous()
+        self._weight_f32 = None
+
+    def add_output(self, y, residual, scale=None, want_cast=False):
+        """`residual += y / rms(y) * weight (* scale)`: the norm on a sublayer's output."""
+        assert self.weight is not None, "RMSNorm used before its weight was loaded"
+        if self._weight_f32 is None:
+            self._weight_f32 = self.weight.float().contiguous()
+        by_column = self._weight_f32 if scale is None else self._weight_f32 * scale
+        return ops.norm_scale_add(y, residual, None, by_column, self.eps, want_cast)
 
     def forward(
         self,
@@ -57,4 +68,44 @@ class RMSNorm(Norm):
 
 @register_norm("rms_norm")
 def build_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> RMSNorm:
-    return RMSNorm(int(desc["hidden_size"]), float(desc["eps"]), dtype, device)
+    return RMSNorm(int(desc["hidden_size"]), float(desc["eps"]), dtype, device, name=str(desc.get("name", "weight")))
+
+
+class ScalarGainRMSNorm(Norm):
+    """RMS norm whose weight is ONE number for all columns: `x / sqrt(mean(x^2) + eps) * gain`.
+
+    As a final norm (`forward`) it runs the row-wise norm kernel with the gain spread over the
+    columns; on a sublayer's output (`add_output`) the one-number form is a kernel argument.
+    The gain stays float32."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, eps: float, dtype: torch.dtype, device, name: str = "weight") -> None:
+        super().__init__(dtype, device)
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+        self.name = name
+        self.gain: torch.Tensor | None = None  # float32 [1]
+        self._spread: torch.Tensor | None = None  # the gain as a weight row in the compute dtype
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {prefix + self.name: ParamSpec((), init="norm_weight", dtype="float32")}
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.gain = get(prefix + self.name).reshape(1).float().contiguous()
+        self._spread = self.gain.to(self.dtype).expand(self.hidden_size).contiguous()
+
+    def forward(self, delta, residual, rows=None):
+        assert self._spread is not None, "norm used before its gain was loaded"
+        if delta is not None and hasattr(delta, "finish"):
+            delta = delta.finish()
+        return ops.add_rmsnorm(delta, residual, self._spread, self.eps, rows)
+
+    def add_output(self, y, residual, scale=None, want_cast=False):
+        assert self.gain is not None, "norm used before its gain was loaded"
+        return ops.norm_scale_add(y, residual, self.gain, scale, self.eps, want_cast)
+
+
+@register_norm("scalar_rms_norm")
+def build_scalar_rms_norm(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ScalarGainRMSNorm:
+    return ScalarGainRMSNorm(int(desc["hidden_size"]), float(desc["eps"]), dtype, device, name=str(desc.get("name", "weight")))

@@ -40,7 +40,7 @@ def random_tensors(
             values = std * values
         else:
             raise ValueError(f"{name}: unknown init {spec.init!r}")
-        tensor = torch.from_numpy(np.ascontiguousarray(values, dtype=np.float32))
+        tensor = torch.from_numpy(np.ascontiguousarray(values, dtype=np.float32)).reshape(spec.shape)
         store = torch.float32 if spec.dtype == "float32" else dtype
         out[name] = tensor.to(store)
     return out
