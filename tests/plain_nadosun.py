@@ -54,21 +54,27 @@ def embedding(table: np.ndarray, tokens: np.ndarray, scale: float, first_positio
     return table[tokens].astype(np.float64) * scale + sinusoid(positions, table.shape[1])
 
 
+def gated_recurrence(z_in, u, gate, state=None):
+    """S_t = (1 - z_t) S_(t-1) + z_t c_t, token by token, from the gates' inputs (biases already
+    added).  Returns (S_t * silu(gate_t) for every t, the last S)."""
+    z = sigmoid(z_in)
+    candidate = np.where(u >= 0, u + 0.5, sigmoid(u))
+    s = np.zeros(z.shape[1]) if state is None else np.array(state, dtype=np.float64)
+    rows = []
+    for t in range(z.shape[0]):
+        s = (1.0 - z[t]) * s + z[t] * candidate[t]
+        rows.append(s * silu(gate[t]))
+    return np.array(rows).reshape(z.shape[0], -1), s
+
+
 def min_gru(h, w, prefix, state=None, store=_same):
-    """The gated recurrence over the rows of h, token by token.  Returns (output rows, last state)."""
+    """The gated recurrence over the rows of h.  Returns (output rows, last state)."""
     f = lambda name: w[prefix + name].astype(np.float64)  # noqa: E731
     z_in = store(h @ f("z").T) + f("z.b")
     u = store(h @ f("x").T) + f("x.b")
     gate = store(h @ f("g").T)
-    z = sigmoid(z_in)
-    candidate = np.where(u >= 0, u + 0.5, sigmoid(u))
-    s = np.zeros(z.shape[1]) if state is None else state.copy()
-    rows = []
-    for t in range(h.shape[0]):
-        s = (1.0 - z[t]) * s + z[t] * candidate[t]
-        rows.append(s * silu(gate[t]))
-    mixed = store(np.array(rows).reshape(h.shape[0], -1))
-    return store(mixed @ f("o").T), s
+    rows, s = gated_recurrence(z_in, u, gate, state)
+    return store(store(rows) @ f("o").T), s
 
 
 def windowed_attention(h, w, prefix, mixer, eps, store=_same, past_k=None, past_v=None):
