@@ -412,6 +412,123 @@ def measure_long_context(contexts: list[int], batch: int, dtype: str, sizes: str
     }
 
 
+# ---------------------------------------------------------------------------------------------
+# --design: another model design beside Llama at equal layer sizes
+# ---------------------------------------------------------------------------------------------
+
+DESIGN_WINDOW = 1024
+DESIGN_LAYERS = 12
+
+
+def nadosun_config(sizes: dict, layers: int) -> dict:
+    """A Nadosun model with the widths of a Llama configuration: two minGRU layers, then a windowed
+    attention layer with a feed-forward, and so on; state as wide as the stream, a window of 1,024 keys."""
+    h = sizes["hidden_size"]
+    attention = {"type": "attention", "mixer": {"heads": sizes["num_attention_heads"], "kv_heads": sizes["num_key_value_heads"],
+                                                "dim": sizes["head_dim"], "vdim": sizes["head_dim"],
+                                                "mask": {"size": DESIGN_WINDOW}, "scale": sizes["head_dim"] ** -0.5},
+                 "mlp": {"kind": "dense", "ff": sizes["intermediate_size"]}}
+    recurrent = {"type": "mingru", "mixer": {"width": h}, "mlp": None}
+    return {"architecture": "Nadosun", "vocab": sizes["vocab_size"], "width": h, "embedding": {"scale": float(h) ** 0.5},
+            "norm": {"eps": 1e-6}, "token_side": {"dim": max(8, h // 16)},
+            "layers": [attention if i % 3 == 2 else recurrent for i in range(layers)]}
+
+
+def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
+    """What a step must move and compute, from the model's own list of tensors: bytes of every matrix
+    a decode step streams (tables that are only gathered from are left out), multiply-adds of its
+    products per token, and per layer kind what attention reads and computes at `context` keys."""
+    gathered = {"embed", "side.embed", "model.embed_tokens.weight"}
+    specs = model.param_specs()
+    matrix = sum(int(s.shape[0]) * int(s.shape[1]) for n, s in specs.items() if len(s.shape) == 2 and n not in gathered)
+    if "lm_head.weight" not in specs and "head" not in specs:  # a tied head streams the embedding's table
+        matrix += int(specs["model.embed_tokens.weight"].shape[0]) * int(specs["model.embed_tokens.weight"].shape[1])
+    head = int(model.vocab_size) * int(model.spec.hidden_size)
+    if "layers" in raw:  # Nadosun: windowed layers
+        layers = [(m["heads"], m["kv_heads"], m["dim"], m["mask"]["size"]) for m in (l["mixer"] for l in raw["layers"] if l["type"] == "attention")]
+    else:
+        layers = [(raw["num_attention_heads"], raw["num_key_value_heads"], raw["head_dim"], None)] * raw["num_hidden_layers"]
+    kv_values = sum(2 * kv * d * (context if w is None else min(context, w)) for _, kv, d, w in layers)
+    pairs = lambda w: sum(min(i + 1, w or tokens) for i in range(tokens))  # noqa: E731
+    attention_flops = sum(4.0 * pairs(w) * d * hq for hq, _, d, w in layers)
+    return {"matrix_values": matrix, "kv_values_per_request": kv_values,
+            "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops}
+
+
+def measure_model(raw: dict, dtype: str, batches: list[int], steps: int, warmup: int) -> dict:
+    """Prefill of one 2,048-token prompt and decode steps at each batch size for any registered design."""
+    import numpy as np
+    import torch
+
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.sampling import sample_from_slots
+
+    elem = 2 if dtype == "bfloat16" else 4
+    pages = -(-(PROMPT_LEN + warmup + steps + 1) // BLOCK_SIZE)
+    runner = ModelRunner.from_random(raw, seed=0, dtype=dtype, num_blocks=max(batches) * pages + 8, block_size=BLOCK_SIZE,
+                                     max_concurrent=max(batches))
+    vocab = runner.vocab_size
+    rng = np.random.default_rng(0)
+    times = []
+    for rep in range(4):
+        prompt = rng.integers(0, vocab, size=PROMPT_LEN).tolist()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        runner.step([StepEntry(f"p{rep}", prompt, [PROMPT_LEN - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - started)
+        runner.free_request(f"p{rep}")
+    seconds = min(times[1:])
+    context = PROMPT_LEN + warmup + (steps + 1) / 2
+    costs = model_costs(runner.model, raw, PROMPT_LEN, context)
+    peak = PEAK_FLOPS["bf16" if dtype == "bfloat16" else "fp32"]
+    out = {"matrix_bytes": costs["matrix_values"] * elem,
+           "prefill": {"tokens": PROMPT_LEN, "ms": round(seconds * 1e3, 3), "tok_s": round(PROMPT_LEN / seconds, 1),
+                       "frac_of_matrix_peak": round(costs["prefill_flops"] / seconds / peak, 4)},
+           "decode": {}}
+    for batch in batches:
+        ids = [f"b{batch}_{i}" for i in range(batch)]
+        for rid in ids:
+            runner.step([StepEntry(rid, rng.integers(0, vocab, size=PROMPT_LEN).tolist(), [PROMPT_LEN - 1])])
+        on_device = None
+        for k in range(warmup + steps):
+            if k == warmup:
+                torch.cuda.synchronize()
+                started = time.perf_counter()
+            if on_device is None:
+                entries = [StepEntry(rid, [1], [0]) for rid in ids]
+            else:
+                entries = [StepEntry(rid, [0], [0], device_row=row) for row, rid in enumerate(ids)]
+            logits = runner.step(entries, device_tokens=on_device)
+            on_device = sample_from_slots(logits, runner.last_row_slots, runner.cache.states.table)
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - started) / steps
+        for rid in ids:
+            runner.free_request(rid)
+        moved = (costs["matrix_values"] + batch * costs["kv_values_per_request"]) * elem
+        out["decode"][f"b{batch}"] = {"ms_per_step": round(seconds * 1e3, 4), "tok_s": round(batch / seconds, 1),
+                                      "frac_of_hbm_peak": round(moved / seconds / 1e9 / PEAK_HBM_GBS, 4)}
+    del runner
+    torch.cuda.empty_cache()
+    return out
+
+
+def measure_design(design: str, sizes_name: str, dtype: str, layers: int | None, batches: list[int], steps: int, warmup: int,
+                   alone: bool = False) -> dict:
+    model_name, sizes = SIZES[sizes_name]
+    layers = layers if layers is not None else DESIGN_LAYERS
+    if design != "nadosun":
+        raise ValueError(f"no design {design!r} to compare")
+    ours = nadosun_config(sizes, layers)
+    theirs = dict(sizes, num_hidden_layers=layers)
+    line = {"design": design, "sizes": f"{model_name} layer sizes", "layers": layers, "dtype": dtype, "window": DESIGN_WINDOW,
+            "data": "synthetic: random token ids, random-init weights", "steps": steps, "warmup": warmup}
+    for name, raw in ((design, ours), ("llama", theirs))[: 1 if alone else 2]:
+        print(f"bench.py: {name} at {model_name} layer sizes, {layers} layers", file=sys.stderr, flush=True)
+        line[name] = measure_model(raw, dtype, batches, steps, warmup)
+    return line
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -448,6 +565,13 @@ def main() -> int:
     parser.add_argument("--no-mixed-graphs", action="store_true",
                         help="with --serving / --reference-workload: launch steps that have portions of prompts in them kernel "
                         "by kernel, however few their tokens (recorded steps of single tokens stay)")
+    parser.add_argument(
+        "--design", default=None, choices=("nadosun",),
+        help="instead of the default run: prefill (one 2,048-token prompt) and decode (batch 1, --batch and 64; --steps "
+        "steps, default 64 here) of that design beside Llama at the layer sizes of --sizes and equal depth "
+        "(--layers, default 12); prints one JSON line and exits",
+    )
+    parser.add_argument("--design-alone", action="store_true", help="with --design: leave the Llama side out (for profiles)")
     parser.add_argument("--attention-batch", type=int, default=0)
     parser.add_argument("--attention-repeats", type=int, default=20)
     args = parser.parse_args()
@@ -457,6 +581,11 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design is not None:
+        steps = args.steps if args.steps != PROMPT_LEN - 8 else 64
+        batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+        print(json.dumps(measure_design(args.design, args.sizes, args.dtype, args.layers, batches, steps, args.warmup, args.design_alone)), flush=True)
+        return 0
     if args.long_context is not None:
         contexts = [int(c) for c in args.long_context.split(",")]
         print(json.dumps(measure_long_context(contexts, args.batch, args.dtype, args.sizes, args.layers)), flush=True)

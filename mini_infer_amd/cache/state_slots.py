@@ -14,7 +14,9 @@ admits and frees a request as a whole.  A slot is
     are advanced by the same events, so they agree whenever the device is idle;
   * one row in each state tensor a mixer asked for, `[max_requests + 1, *shape]` per
     layer call (several per call, each of its own shape and dtype, where the mixer named
-    several), zeroed when the slot is handed out (Llama asks for none).  The last
+    several), zeroed when the slot is handed out (Llama asks for none).  The tensors are views
+    into one buffer per dtype, so rows of different slots are `stride(0)` elements apart, which
+    is more than the row's own size: kernels take that stride as an argument.  The last
     row belongs to no request: the padding rows of a recorded decode step carry slot
     -1, which indexes it, so a mixer that reads and writes `state[slots]` with device
     tensors alone needs no special case for them and can be recorded.
@@ -55,6 +57,7 @@ def _as_i32(value: int) -> int:
 
 
 STAGING_ROWS = 64  # pinned rows a slot-table row waits in for its copy to the device
+STATE_COLUMN_STEP = 64  # a need's columns in the shared state buffer start at a multiple of this many elements
 
 
 class StateSlots:
@@ -88,16 +91,32 @@ class StateSlots:
                 self._staging = torch.empty((STAGING_ROWS, SLOT_WORDS), dtype=torch.int32, pin_memory=True)
                 self._staging_events = [None] * STAGING_ROWS
 
-            def make(need: StateNeeds) -> torch.Tensor:
-                tensor = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
-                self._all_tensors.append(tensor)
-                return tensor
-
+            # All state of one dtype lies in ONE buffer [max_requests + 1, columns]; a need's tensor is
+            # the view of its columns (each need starts on a 256-byte boundary).  Zeroing a slot's
+            # state, and copying a step's rows aside and back, then touch one tensor per dtype
+            # whatever the number of layers (a model of a dozen recurrent layers measured 32 small
+            # launches a step for the copies alone when every layer had a tensor of its own).
+            layout: list[tuple[int, str | None, StateNeeds, int, int]] = []
+            columns: dict[torch.dtype, int] = {}
             for call, need in needs.items():
-                if isinstance(need, StateNeeds):
-                    self.tensors[call] = make(need)
+                for name, one in ([(None, need)] if isinstance(need, StateNeeds) else list(need.items())):
+                    count = 1
+                    for extent in one.shape:
+                        count *= int(extent)
+                    at = columns.get(one.dtype, 0)
+                    layout.append((call, name, one, at, count))
+                    columns[one.dtype] = at + -(-count // STATE_COLUMN_STEP) * STATE_COLUMN_STEP
+            buffers = {
+                dtype: torch.zeros((max_requests + 1, total), dtype=dtype, device=device) for dtype, total in columns.items()
+            }
+            self._all_tensors = list(buffers.values())
+            for call, name, one, at, count in layout:
+                view = buffers[one.dtype][:, at : at + count]
+                view = view.unflatten(1, tuple(one.shape)) if len(one.shape) > 0 else view[:, 0]
+                if name is None:
+                    self.tensors[call] = view
                 else:
-                    self.tensors[call] = {name: make(one) for name, one in need.items()}
+                    self.tensors.setdefault(call, {})[name] = view  # type: ignore[union-attr]
 
     @property
     def num_free(self) -> int:
@@ -129,12 +148,14 @@ class StateSlots:
         nobody's row), one per state tensor: what `restore` puts back when the step that was
         about to update them fails."""
         index = slots.long()
-        return [tensor.index_select(0, torch.where(index < 0, index + tensor.shape[0], index)) for tensor in self._all_tensors]
+        rows = torch.where(index < 0, index + (self.max_requests + 1), index)
+        return [tensor.index_select(0, rows) for tensor in self._all_tensors]
 
     def restore(self, slots: torch.Tensor, saved: list[torch.Tensor]) -> None:
         index = slots.long()
+        at = torch.where(index < 0, index + (self.max_requests + 1), index)
         for tensor, rows in zip(self._all_tensors, saved):
-            tensor.index_copy_(0, torch.where(index < 0, index + tensor.shape[0], index), rows)
+            tensor.index_copy_(0, at, rows)
 
     def free(self, slot: int) -> None:
         if not 0 <= slot < self.max_requests:

@@ -15,6 +15,30 @@
 
 #include <math.h>
 
+typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+
+// four consecutive elements at once (8- and 16-byte accesses; the caller checks alignment)
+__device__ __forceinline__ void load4(const float* p, float v[4]) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float v[4]) {
+  const bf16x4_t x = *reinterpret_cast<const bf16x4_t*>(p);
+  v[0] = (float)x[0]; v[1] = (float)x[1]; v[2] = (float)x[2]; v[3] = (float)x[3];
+}
+__device__ __forceinline__ void store4(float* p, const float v[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float v[4]) {
+  bf16x4_t x;
+  x[0] = (bf16_t)v[0]; x[1] = (bf16_t)v[1]; x[2] = (bf16_t)v[2]; x[3] = (bf16_t)v[3];
+  *reinterpret_cast<bf16x4_t*>(p) = x;
+}
+static inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+// Row kernels run one block a row: few rows (decode) get wide blocks so that a row is one or two
+// trips a thread, many rows (prompts) narrow ones so that several rows share a CU.
+static inline int row_block(int rows, int items) { return (rows < 256 && items > 1024) ? 1024 : 256; }
+
 template <typename T>
 struct Wide {
   using type = float;
@@ -61,17 +85,15 @@ __global__ __launch_bounds__(256) void embed_sinusoid_kernel(
     const double* __restrict__ freq, float* __restrict__ residual, T* __restrict__ cast, int hidden, float scale) {
   using A = typename Wide<T>::type;
   const int t = blockIdx.x;
-  const T* row = table + (int64_t)ids[t] * hidden;
-  const A pos = (A)positions[t];
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const A angle = pos * (A)freq[i / 2];
-    A wave;
-    if constexpr (sizeof(T) == 4) wave = (i & 1) ? cos(angle) : sin(angle);
-    else wave = (i & 1) ? cosf(angle) : sinf(angle);
-    const float v = (float)((A)to_f32(row[i]) * (A)scale + wave);
-    residual[(int64_t)t * hidden + i] = v;
-    if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(v);
-  }
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;  // the blocks along y share a token's columns
+  if (i >= hidden) return;
+  const A angle = (A)positions[t] * (A)freq[i / 2];
+  A wave;
+  if constexpr (sizeof(T) == 4) wave = (i & 1) ? cos(angle) : sin(angle);
+  else wave = (i & 1) ? cosf(angle) : sinf(angle);
+  const float v = (float)((A)to_f32(table[(int64_t)ids[t] * hidden + i]) * (A)scale + wave);
+  residual[(int64_t)t * hidden + i] = v;
+  if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(v);
 }
 
 extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, const int* positions,
@@ -81,11 +103,13 @@ extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, c
              num_tokens, hidden, vocab);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_sinusoid: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  MI_REQUIRE(ceil_div(hidden, 256) <= 65535, "embed_sinusoid: hidden=%d is too wide for one launch", hidden);
+  const dim3 grid(num_tokens, ceil_div(hidden, 256));
   if (dtype == MI_F32) {
-    embed_sinusoid_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)table, ids, positions, freq, residual,
+    embed_sinusoid_kernel<float><<<grid, 256, 0, stream>>>((const float*)table, ids, positions, freq, residual,
                                                                  (float*)cast, hidden, scale);
   } else {
-    embed_sinusoid_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)table, ids, positions, freq,
+    embed_sinusoid_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)table, ids, positions, freq,
                                                                   residual, (bf16_t*)cast, hidden, scale);
   }
   MI_CHECK_LAUNCH("embed_sinusoid");
@@ -100,29 +124,67 @@ extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, c
 // next sublayer's products read.  One block a row.
 // ---------------------------------------------------------------------------
 
-template <typename T>
-__global__ __launch_bounds__(256) void norm_scale_add_kernel(
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void norm_scale_add_kernel(
     const T* __restrict__ y, int64_t y_stride, float* __restrict__ residual, const float* __restrict__ gain,
     const float* __restrict__ scale, T* __restrict__ cast, int hidden, float eps) {
   using A = typename Wide<T>::type;
-  __shared__ A scratch[4];
+  __shared__ A scratch[16];
   const int t = blockIdx.x;
   const T* row = y + (int64_t)t * y_stride;
   A squares = 0;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const A v = (A)to_f32(row[i]);
-    squares += v * v;
+  for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
+    float v[VEC];
+    if constexpr (VEC == 4) load4(row + i, v);
+    else v[0] = to_f32(row[i]);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) squares += (A)v[k] * (A)v[k];
   }
   const A inv = inv_root(block_total<A>(squares, scratch) / (A)hidden, (A)eps);
   const A g = gain != nullptr ? (A)gain[0] : (A)1;
   float* res = residual + (int64_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    A v = ((A)to_f32(row[i]) * inv) * g;
-    if (scale != nullptr) v *= (A)scale[i];
-    const float sum = (float)((A)res[i] + v);
-    res[i] = sum;
-    if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(sum);
+  for (int i = threadIdx.x * VEC; i < hidden; i += blockDim.x * VEC) {
+    float v[VEC], r[VEC], sc[VEC];
+    if constexpr (VEC == 4) {
+      load4(row + i, v);
+      load4(res + i, r);
+      if (scale != nullptr) load4(scale + i, sc);
+    } else {
+      v[0] = to_f32(row[i]);
+      r[0] = res[i];
+      if (scale != nullptr) sc[0] = scale[i];
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      A add = ((A)v[k] * inv) * g;
+      if (scale != nullptr) add *= (A)sc[k];
+      r[k] = (float)((A)r[k] + add);
+    }
+    if constexpr (VEC == 4) {
+      store4(res + i, r);
+      if (cast != nullptr) store4(cast + (int64_t)t * hidden + i, r);
+    } else {
+      res[i] = r[0];
+      if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(r[0]);
+    }
   }
+}
+
+template <typename T>
+static int norm_scale_add_launch(const void* y, int64_t y_stride, float* residual, const float* gain, const float* scale,
+                                 void* cast, int num_tokens, int hidden, float eps, hipStream_t stream) {
+  const bool vec = hidden % 4 == 0 && y_stride % 4 == 0 && aligned16(y) && aligned16(residual) && aligned16(scale) &&
+                   aligned16(cast) && (sizeof(T) == 4 || y_stride % 8 == 0);
+  const int threads = row_block(num_tokens, vec ? hidden / 4 : hidden);
+  if (vec) {
+    norm_scale_add_kernel<T, 4><<<num_tokens, threads, 0, stream>>>((const T*)y, y_stride, residual, gain, scale, (T*)cast,
+                                                                hidden, eps);
+  } else {
+    norm_scale_add_kernel<T, 1><<<num_tokens, threads, 0, stream>>>((const T*)y, y_stride, residual, gain, scale, (T*)cast,
+                                                                hidden, eps);
+  }
+  MI_CHECK_LAUNCH("norm_scale_add");
+  return MI_OK;
 }
 
 extern "C" int mi_norm_scale_add(int dtype, const void* y, int64_t y_stride, float* residual, const float* gain,
@@ -132,15 +194,8 @@ extern "C" int mi_norm_scale_add(int dtype, const void* y, int64_t y_stride, flo
              num_tokens, hidden, (long long)y_stride);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "norm_scale_add: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
-  if (dtype == MI_F32) {
-    norm_scale_add_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)y, y_stride, residual, gain, scale,
-                                                                 (float*)cast, hidden, eps);
-  } else {
-    norm_scale_add_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)y, y_stride, residual, gain, scale,
-                                                                  (bf16_t*)cast, hidden, eps);
-  }
-  MI_CHECK_LAUNCH("norm_scale_add");
-  return MI_OK;
+  if (dtype == MI_F32) return norm_scale_add_launch<float>(y, y_stride, residual, gain, scale, cast, num_tokens, hidden, eps, stream);
+  return norm_scale_add_launch<bf16_t>(y, y_stride, residual, gain, scale, cast, num_tokens, hidden, eps, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -180,33 +235,63 @@ __device__ __forceinline__ void gru_gates(A z_in, A u, A& keep, A& add) {
   add = z * cand;
 }
 
-template <typename T>
+// VEC consecutive columns of a row, as float
+template <typename T, int VEC>
+__device__ __forceinline__ void load_cols(const T* p, float v[VEC]) {
+  if constexpr (VEC == 4) load4(p, v);
+  else v[0] = to_f32(p[0]);
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void store_cols(T* p, const float v[VEC]) {
+  if constexpr (VEC == 4) store4(p, v);
+  else p[0] = from_f32<T>(v[0]);
+}
+
+// One step of the recurrence for a thread's VEC columns of row `in`; with `out`, the gated
+// output of the row is written.
+template <typename T, int VEC, bool SUMMARY, typename A>
+__device__ __forceinline__ void gru_row(const T* __restrict__ in, int width, int c, const A* bias_z, const A* bias_x,
+                                        A* s, A* p, T* __restrict__ out) {
+  float z_in[VEC], u[VEC], g[VEC], y[VEC];
+  load_cols<T, VEC>(in + c, z_in);
+  load_cols<T, VEC>(in + width + c, u);
+  if constexpr (!SUMMARY) load_cols<T, VEC>(in + 2 * (int64_t)width + c, g);
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    A keep, add;
+    gru_gates<A>((A)z_in[k] + bias_z[k], (A)u[k] + bias_x[k], keep, add);
+    s[k] = keep * s[k] + add;
+    if constexpr (SUMMARY) p[k] *= keep;
+    else y[k] = (float)(s[k] * ((A)g[k] * logistic((A)g[k])));
+  }
+  if constexpr (!SUMMARY) store_cols<T, VEC>(out + c, y);
+}
+
+template <typename T, int VEC>
 __global__ __launch_bounds__(64) void gated_scan_kernel(
     const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
-    float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ out,
-    int64_t out_stride, int width, int num_slots) {
+    float* __restrict__ state, int64_t state_stride, const int* __restrict__ cu, const int* __restrict__ slots,
+    T* __restrict__ out, int64_t out_stride, int width, int num_slots) {
   using A = typename Wide<T>::type;
   const int b = blockIdx.y;
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (c >= width) return;
   const int first = cu[b], last = cu[b + 1];
   if (last <= first) return;
   const int slot = slots[b];
-  const int64_t row = (slot < 0 || slot >= num_slots) ? num_slots : slot;
-  A s = (A)state[row * width + c];
-  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
-#pragma unroll 4
-  for (int t = first; t < last; ++t) {
-    const T* in = zxg + (int64_t)t * in_stride;
-    const A z_in = (A)to_f32(in[c]) + bias_z;
-    const A u = (A)to_f32(in[width + c]) + bias_x;
-    const A g = (A)to_f32(in[2 * (int64_t)width + c]);
-    A keep, add;
-    gru_gates<A>(z_in, u, keep, add);
-    s = keep * s + add;
-    out[(int64_t)t * out_stride + c] = from_f32<T>((float)(s * (g * logistic(g))));
+  float* mine = state + ((slot < 0 || slot >= num_slots) ? num_slots : slot) * state_stride + c;
+  A s[VEC], bias_z[VEC], bias_x[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    s[k] = (A)mine[k];
+    bias_z[k] = (A)bz[c + k];
+    bias_x[k] = (A)bx[c + k];
   }
-  state[row * width + c] = (float)s;
+#pragma unroll 4
+  for (int t = first; t < last; ++t)
+    gru_row<T, VEC, false, A>(zxg + (int64_t)t * in_stride, width, c, bias_z, bias_x, s, nullptr, out + (int64_t)t * out_stride);
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) mine[k] = (float)s[k];
 }
 
 // Chunked form for long portions: the recurrence S' = keep * S + add is linear in S, so a
@@ -215,35 +300,42 @@ __global__ __launch_bounds__(64) void gated_scan_kernel(
 // walks each request's chunks in order and leaves every chunk's incoming state, pass 3 redoes
 // every chunk from its incoming state and writes the outputs.  Chunks are cut per request
 // at multiples of `chunk` rows from the request's first row of the step.
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(64) void gated_scan_summaries_kernel(
     const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
     const int* __restrict__ cu, float* __restrict__ summaries, int width, int chunk, int chunks_per_request) {
   using A = typename Wide<T>::type;
   const int b = blockIdx.z, k = blockIdx.y;
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (c >= width) return;
   const int first = cu[b] + k * chunk, last = min(cu[b + 1], first + chunk);
   if (last <= first) return;
-  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
-  A p = 1, q = 0;
-#pragma unroll 4
-  for (int t = first; t < last; ++t) {
-    const T* in = zxg + (int64_t)t * in_stride;
-    A keep, add;
-    gru_gates<A>((A)to_f32(in[c]) + bias_z, (A)to_f32(in[width + c]) + bias_x, keep, add);
-    p *= keep;
-    q = keep * q + add;
+  A p[VEC], q[VEC], bias_z[VEC], bias_x[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    p[j] = 1;
+    q[j] = 0;
+    bias_z[j] = (A)bz[c + j];
+    bias_x[j] = (A)bx[c + j];
   }
+#pragma unroll 8
+  for (int t = first; t < last; ++t)
+    gru_row<T, VEC, true, A>(zxg + (int64_t)t * in_stride, width, c, bias_z, bias_x, q, p, nullptr);
   float* at = summaries + (((int64_t)b * chunks_per_request + k) * 2) * width;
-  at[c] = (float)p;
-  at[width + c] = (float)q;
+  float pf[VEC], qf[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    pf[j] = (float)p[j];
+    qf[j] = (float)q[j];
+  }
+  store_cols<float, VEC>(at + c, pf);
+  store_cols<float, VEC>(at + width + c, qf);
 }
 
 // Pass 2: every chunk's (P, Q) is replaced by its incoming state (in Q's place); the request's
 // state row receives the state after its last row.
 __global__ __launch_bounds__(64) void gated_scan_carry_kernel(
-    float* __restrict__ summaries, float* __restrict__ state, const int* __restrict__ cu,
+    float* __restrict__ summaries, float* __restrict__ state, int64_t state_stride, const int* __restrict__ cu,
     const int* __restrict__ slots, int width, int chunk, int chunks_per_request, int num_slots) {
   const int b = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -251,88 +343,100 @@ __global__ __launch_bounds__(64) void gated_scan_carry_kernel(
   const int rows = cu[b + 1] - cu[b];
   if (rows <= 0) return;
   const int slot = slots[b];
-  const int64_t row = (slot < 0 || slot >= num_slots) ? num_slots : slot;
+  float* mine = state + ((slot < 0 || slot >= num_slots) ? num_slots : slot) * state_stride + c;
   const int chunks = (rows + chunk - 1) / chunk;
-  float s = state[row * width + c];
+  float s = *mine;
+#pragma unroll 8
   for (int k = 0; k < chunks; ++k) {
     float* at = summaries + (((int64_t)b * chunks_per_request + k) * 2) * width;
     const float p = at[c], q = at[width + c];
     at[width + c] = s;
     s = p * s + q;
   }
-  state[row * width + c] = s;
+  *mine = s;
 }
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(64) void gated_scan_outputs_kernel(
     const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
     const int* __restrict__ cu, const float* __restrict__ summaries, T* __restrict__ out, int64_t out_stride,
     int width, int chunk, int chunks_per_request) {
   using A = typename Wide<T>::type;
   const int b = blockIdx.z, k = blockIdx.y;
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (c >= width) return;
   const int first = cu[b] + k * chunk, last = min(cu[b + 1], first + chunk);
   if (last <= first) return;
-  const A bias_z = (A)bz[c], bias_x = (A)bx[c];
-  A s = (A)summaries[(((int64_t)b * chunks_per_request + k) * 2 + 1) * width + c];
-#pragma unroll 4
-  for (int t = first; t < last; ++t) {
-    const T* in = zxg + (int64_t)t * in_stride;
-    const A g = (A)to_f32(in[2 * (int64_t)width + c]);
-    A keep, add;
-    gru_gates<A>((A)to_f32(in[c]) + bias_z, (A)to_f32(in[width + c]) + bias_x, keep, add);
-    s = keep * s + add;
-    out[(int64_t)t * out_stride + c] = from_f32<T>((float)(s * (g * logistic(g))));
+  A s[VEC], bias_z[VEC], bias_x[VEC];
+  float incoming[VEC];
+  load_cols<float, VEC>(summaries + (((int64_t)b * chunks_per_request + k) * 2 + 1) * width + c, incoming);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    s[j] = (A)incoming[j];
+    bias_z[j] = (A)bz[c + j];
+    bias_x[j] = (A)bx[c + j];
   }
+#pragma unroll 8
+  for (int t = first; t < last; ++t)
+    gru_row<T, VEC, false, A>(zxg + (int64_t)t * in_stride, width, c, bias_z, bias_x, s, nullptr, out + (int64_t)t * out_stride);
 }
 
-template <typename T>
+template <typename T, int VEC>
 static int gated_scan_launch(const void* zxg, int64_t in_stride, const float* bz, const float* bx, float* state,
-                             const int* cu, const int* slots, void* out, int64_t out_stride, int num_requests,
-                             int width, int num_slots, int chunk, int chunks_per_request, float* summaries,
-                             hipStream_t stream) {
-  const int col_blocks = ceil_div(width, 64);
+                             int64_t state_stride, const int* cu, const int* slots, void* out, int64_t out_stride,
+                             int num_requests, int width, int num_slots, int chunk, int chunks_per_request,
+                             float* summaries, hipStream_t stream) {
+  const int col_blocks = ceil_div(ceil_div(width, VEC), 64);
   if (chunk <= 0) {
     dim3 grid(col_blocks, num_requests);
-    gated_scan_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, state, cu, slots, (T*)out,
-                                                  out_stride, width, num_slots);
+    gated_scan_kernel<T, VEC><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, state, state_stride, cu, slots,
+                                                       (T*)out, out_stride, width, num_slots);
     MI_CHECK_LAUNCH("gated_scan");
     return MI_OK;
   }
   dim3 grid(col_blocks, chunks_per_request, num_requests);
-  gated_scan_summaries_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, width,
-                                                          chunk, chunks_per_request);
+  gated_scan_summaries_kernel<T, VEC><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, width,
+                                                               chunk, chunks_per_request);
   MI_CHECK_LAUNCH("gated_scan (summaries)");
-  gated_scan_carry_kernel<<<dim3(col_blocks, num_requests), 64, 0, stream>>>(summaries, state, cu, slots, width, chunk,
-                                                                             chunks_per_request, num_slots);
+  gated_scan_carry_kernel<<<dim3(ceil_div(width, 64), num_requests), 64, 0, stream>>>(
+      summaries, state, state_stride, cu, slots, width, chunk, chunks_per_request, num_slots);
   MI_CHECK_LAUNCH("gated_scan (carry)");
-  gated_scan_outputs_kernel<T><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, (T*)out,
-                                                        out_stride, width, chunk, chunks_per_request);
+  gated_scan_outputs_kernel<T, VEC><<<grid, 64, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, (T*)out,
+                                                             out_stride, width, chunk, chunks_per_request);
   MI_CHECK_LAUNCH("gated_scan (outputs)");
   return MI_OK;
 }
 
 // `chunk` = 0: the sequential form.  `chunk` > 0: the chunked form; no request may bring more
 // than chunk * chunks_per_request rows (the caller's bound), and `summaries` holds
-// num_requests * chunks_per_request * 2 * width floats.
+// num_requests * chunks_per_request * 2 * width floats.  `state_stride`: floats between the
+// state rows of two slots.
 extern "C" int mi_gated_scan(int dtype, const void* zxg, int64_t in_stride, const float* bz, const float* bx,
-                             float* state, const int* cu, const int* slots, void* out, int64_t out_stride,
-                             int num_requests, int width, int num_slots, int chunk, int chunks_per_request,
-                             float* summaries, hipStream_t stream) {
+                             float* state, int64_t state_stride, const int* cu, const int* slots, void* out,
+                             int64_t out_stride, int num_requests, int width, int num_slots, int chunk,
+                             int chunks_per_request, float* summaries, hipStream_t stream) {
   MI_REQUIRE(num_requests >= 0 && width > 0 && num_slots >= 0, "gated_scan: bad sizes requests=%d width=%d slots=%d",
              num_requests, width, num_slots);
-  MI_REQUIRE(in_stride >= 3 * (int64_t)width && out_stride >= width, "gated_scan: rows hold [z | x | g], %d each", width);
+  MI_REQUIRE(in_stride >= 3 * (int64_t)width && out_stride >= width && state_stride >= width,
+             "gated_scan: rows hold [z | x | g], %d each", width);
   MI_REQUIRE(chunk >= 0 && (chunk == 0 || (chunks_per_request > 0 && summaries != nullptr)),
              "gated_scan: the chunked form needs a chunk count and a summaries buffer");
   MI_REQUIRE(num_requests <= 65535 && chunks_per_request <= 65535, "gated_scan: too many requests or chunks for one launch");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "gated_scan: unknown dtype %d", dtype);
   if (num_requests == 0) return MI_OK;
-  if (dtype == MI_F32)
-    return gated_scan_launch<float>(zxg, in_stride, bz, bx, state, cu, slots, out, out_stride, num_requests, width,
-                                    num_slots, chunk, chunks_per_request, summaries, stream);
-  return gated_scan_launch<bf16_t>(zxg, in_stride, bz, bx, state, cu, slots, out, out_stride, num_requests, width,
-                                   num_slots, chunk, chunks_per_request, summaries, stream);
+  const int64_t step = dtype == MI_F32 ? 4 : 8;  // elements of a 16-byte boundary
+  const bool vec = width % 4 == 0 && in_stride % step == 0 && out_stride % step == 0 && width % step == 0 &&
+                   aligned16(zxg) && aligned16(out) && aligned16(summaries);
+#define MI_SCAN(T, VEC)                                                                                              \
+  return gated_scan_launch<T, VEC>(zxg, in_stride, bz, bx, state, state_stride, cu, slots, out, out_stride,           \
+                                   num_requests, width, num_slots, chunk, chunks_per_request, summaries, stream)
+  if (dtype == MI_F32) {
+    if (vec) MI_SCAN(float, 4);
+    MI_SCAN(float, 1);
+  }
+  if (vec) MI_SCAN(bf16_t, 4);
+  MI_SCAN(bf16_t, 1);
+#undef MI_SCAN
 }
 
 // ---------------------------------------------------------------------------
@@ -344,39 +448,60 @@ extern "C" int mi_gated_scan(int dtype, const void* zxg, int64_t in_stride, cons
 // Page layouts and slot numbering are those of rope_kv_write.  kv_heads = 0: q only.
 // ---------------------------------------------------------------------------
 
-template <typename T>
-__global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void qk_norm_kv_write_kernel(
     T* __restrict__ qk, int64_t row_stride, const float* __restrict__ qw, const float* __restrict__ kw,
     const int* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int q_width,
     int kv_heads, int head_dim, int page_size, int v_transposed, float eps) {
   using A = typename Wide<T>::type;
-  __shared__ A scratch[4];
+  __shared__ A scratch[16];
   const int t = blockIdx.x;
   T* row = qk + (int64_t)t * row_stride;
   const int k_width = kv_heads * head_dim;
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;
   A q_squares = 0, k_squares = 0;
-  for (int i = threadIdx.x; i < q_width; i += blockDim.x) {
-    const A v = (A)to_f32(row[i]);
-    q_squares += v * v;
+  for (int i = first; i < q_width; i += stride) {
+    float v[VEC];
+    load_cols<T, VEC>(row + i, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) q_squares += (A)v[j] * (A)v[j];
   }
-  for (int i = threadIdx.x; i < k_width; i += blockDim.x) {
-    const A v = (A)to_f32(row[q_width + i]);
-    k_squares += v * v;
+  for (int i = first; i < k_width; i += stride) {
+    float v[VEC];
+    load_cols<T, VEC>(row + q_width + i, v);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) k_squares += (A)v[j] * (A)v[j];
   }
   const A q_inv = inv_root(block_total<A>(q_squares, scratch) / (A)q_width, (A)eps);
-  for (int i = threadIdx.x; i < q_width; i += blockDim.x)
-    row[i] = from_f32<T>((float)(((A)to_f32(row[i]) * q_inv) * (A)qw[i]));
-  if (k_width == 0 || slot_mapping == nullptr) return;
-  const A k_inv = inv_root(block_total<A>(k_squares, scratch) / (A)k_width, (A)eps);
+  const bool writes = k_width > 0 && slot_mapping != nullptr;
+  const A k_inv = writes ? inv_root(block_total<A>(k_squares, scratch) / (A)k_width, (A)eps) : (A)0;
+  for (int i = first; i < q_width; i += stride) {
+    float v[VEC], w[VEC];
+    load_cols<T, VEC>(row + i, v);
+    load_cols<float, VEC>(qw + i, w);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) v[j] = (float)(((A)v[j] * q_inv) * (A)w[j]);
+    store_cols<T, VEC>(row + i, v);
+  }
+  if (!writes) return;
   const int slot = slot_mapping[t];
   if (slot < 0) return;
   const int page = slot / page_size, off = slot % page_size;
-  for (int e = threadIdx.x; e < k_width; e += blockDim.x) {
-    const int h = e / head_dim, d = e % head_dim;
-    const T raw = row[q_width + e];
+  for (int e = first; e < k_width; e += stride) {
+    const int h = e / head_dim, d = e % head_dim;  // (VEC divides head_dim: the VEC values lie in one head)
+    float raw[VEC], w[VEC], normed[VEC];
+    load_cols<T, VEC>(row + q_width + e, raw);
+    load_cols<float, VEC>(kw + e, w);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) normed[j] = (float)(((A)raw[j] * k_inv) * (A)w[j]);
     const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
-    k_pages[chunk + (int64_t)off * head_dim + d] = from_f32<T>((float)(((A)to_f32(raw) * k_inv) * (A)kw[e]));
-    v_pages[v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * head_dim + d] = raw;
+    store_cols<T, VEC>(k_pages + chunk + (int64_t)off * head_dim + d, normed);
+    if (v_transposed) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) v_pages[chunk + (int64_t)(d + j) * page_size + off] = from_f32<T>(raw[j]);
+    } else {
+      store_cols<T, VEC>(v_pages + chunk + (int64_t)off * head_dim + d, raw);
+    }
   }
 }
 
@@ -393,15 +518,22 @@ extern "C" int mi_qk_norm_kv_write(int dtype, void* qk, int64_t row_stride, cons
              "qk_norm_kv_write: pages and the key norm's weight are needed to write keys and values");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "qk_norm_kv_write: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  const int64_t step = dtype == MI_F32 ? 4 : 8;
+  const bool vec = q_width % step == 0 && head_dim % step == 0 && row_stride % step == 0 && aligned16(qk) && aligned16(qw) &&
+                   aligned16(kw) && aligned16(k_pages) && aligned16(v_pages);
+  const int threads = row_block(num_tokens, (q_width + kv_heads * head_dim) / (vec ? 4 : 1));
+#define MI_QK(T, VEC)                                                                                               \
+  qk_norm_kv_write_kernel<T, VEC><<<num_tokens, threads, 0, stream>>>((T*)qk, row_stride, qw, kw, slot_mapping,      \
+                                                                      (T*)k_pages, (T*)v_pages, q_width, kv_heads,   \
+                                                                      head_dim, page_size, v_transposed, eps)
   if (dtype == MI_F32) {
-    qk_norm_kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)qk, row_stride, qw, kw, slot_mapping,
-                                                                   (float*)k_pages, (float*)v_pages, q_width, kv_heads,
-                                                                   head_dim, page_size, v_transposed, eps);
+    if (vec) MI_QK(float, 4);
+    else MI_QK(float, 1);
   } else {
-    qk_norm_kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)qk, row_stride, qw, kw, slot_mapping,
-                                                                    (bf16_t*)k_pages, (bf16_t*)v_pages, q_width,
-                                                                    kv_heads, head_dim, page_size, v_transposed, eps);
+    if (vec) MI_QK(bf16_t, 4);
+    else MI_QK(bf16_t, 1);
   }
+#undef MI_QK
   MI_CHECK_LAUNCH("qk_norm_kv_write");
   return MI_OK;
 }
@@ -412,32 +544,59 @@ extern "C" int mi_qk_norm_kv_write(int dtype, void* qk, int64_t row_stride, cons
 // `coef` = (a, b, c, e) float32.  One block a row.
 // ---------------------------------------------------------------------------
 
-template <typename T>
-__global__ __launch_bounds__(256) void poly_norm_kernel(const T* __restrict__ z, int64_t in_stride,
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void poly_norm_kernel(const T* __restrict__ z, int64_t in_stride,
                                                         const float* __restrict__ coef, T* __restrict__ out,
                                                         int64_t out_stride, int width, float eps) {
   using A = typename Wide<T>::type;
-  __shared__ A scratch[4];
+  __shared__ A scratch[16];
   const int t = blockIdx.x;
   const T* row = z + (int64_t)t * in_stride;
   A s2 = 0, s4 = 0, s6 = 0;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const A v = (A)to_f32(row[i]);
-    const A v2 = v * v;
-    s2 += v2;
-    s4 += v2 * v2;
-    s6 += v2 * v2 * v2;
+  for (int i = threadIdx.x * VEC; i < width; i += blockDim.x * VEC) {
+    float x[VEC];
+    if constexpr (VEC == 4) load4(row + i, x);
+    else x[0] = to_f32(row[i]);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const A v2 = (A)x[k] * (A)x[k];
+      s2 += v2;
+      s4 += v2 * v2;
+      s6 += v2 * v2 * v2;
+    }
   }
   const A n = (A)width;
   const A i1 = inv_root(block_total<A>(s2, scratch) / n, (A)eps);
   const A i2 = inv_root(block_total<A>(s4, scratch) / n, (A)eps);
   const A i3 = inv_root(block_total<A>(s6, scratch) / n, (A)eps);
   const A a = (A)coef[0] * i1, b = (A)coef[1] * i2, c = (A)coef[2] * i3, e = (A)coef[3];
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const A v = (A)to_f32(row[i]);
-    const A v2 = v * v;
-    out[(int64_t)t * out_stride + i] = from_f32<T>((float)(a * v + b * v2 + c * (v2 * v) + e));
+  for (int i = threadIdx.x * VEC; i < width; i += blockDim.x * VEC) {
+    float x[VEC];
+    if constexpr (VEC == 4) load4(row + i, x);
+    else x[0] = to_f32(row[i]);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const A v = (A)x[k], v2 = v * v;
+      x[k] = (float)(a * v + b * v2 + c * (v2 * v) + e);
+    }
+    if constexpr (VEC == 4) store4(out + (int64_t)t * out_stride + i, x);
+    else out[(int64_t)t * out_stride + i] = from_f32<T>(x[0]);
   }
+}
+
+template <typename T>
+static int poly_norm_launch(const void* z, int64_t in_stride, const float* coef, void* out, int64_t out_stride,
+                            int num_tokens, int width, float eps, hipStream_t stream) {
+  const int64_t step = sizeof(T) == 4 ? 4 : 8;
+  const bool vec = width % 4 == 0 && in_stride % step == 0 && out_stride % step == 0 && aligned16(z) && aligned16(out);
+  const int threads = row_block(num_tokens, vec ? width / 4 : width);
+  if (vec) {
+    poly_norm_kernel<T, 4><<<num_tokens, threads, 0, stream>>>((const T*)z, in_stride, coef, (T*)out, out_stride, width, eps);
+  } else {
+    poly_norm_kernel<T, 1><<<num_tokens, threads, 0, stream>>>((const T*)z, in_stride, coef, (T*)out, out_stride, width, eps);
+  }
+  MI_CHECK_LAUNCH("poly_norm");
+  return MI_OK;
 }
 
 extern "C" int mi_poly_norm(int dtype, const void* z, int64_t in_stride, const float* coef, void* out,
@@ -446,15 +605,8 @@ extern "C" int mi_poly_norm(int dtype, const void* z, int64_t in_stride, const f
              "poly_norm: bad sizes tokens=%d width=%d", num_tokens, width);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "poly_norm: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
-  if (dtype == MI_F32) {
-    poly_norm_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)z, in_stride, coef, (float*)out, out_stride,
-                                                            width, eps);
-  } else {
-    poly_norm_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)z, in_stride, coef, (bf16_t*)out,
-                                                             out_stride, width, eps);
-  }
-  MI_CHECK_LAUNCH("poly_norm");
-  return MI_OK;
+  if (dtype == MI_F32) return poly_norm_launch<float>(z, in_stride, coef, out, out_stride, num_tokens, width, eps, stream);
+  return poly_norm_launch<bf16_t>(z, in_stride, coef, out, out_stride, num_tokens, width, eps, stream);
 }
 
 // ---------------------------------------------------------------------------

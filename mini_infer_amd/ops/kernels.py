@@ -1156,7 +1156,7 @@ def cast_rows(residual: torch.Tensor) -> torch.Tensor:
     return out
 
 
-GATED_SCAN_CHUNK = 64  # rows of a chunk of the chunked recurrence
+GATED_SCAN_CHUNK = 32  # rows of a chunk of the chunked recurrence
 GATED_SCAN_SEQUENTIAL_ROWS = 128  # portions up to this many rows are walked by one thread a column
 
 
@@ -1166,11 +1166,11 @@ def gated_scan(
 ) -> torch.Tensor:
     """minGRU over the rows of a step.  `zxg` [T, 3W] holds the projections [z | x | g] of every
     token; request b owns rows `cu_seqlens[b]..cu_seqlens[b+1]` and the state row `state[slots[b]]`
-    (float32 [slots + 1, W]; a negative slot means the last row, which is nobody's).  Returns
+    (float32 [slots + 1, W], rows may be strided; a negative slot means the last row, which is nobody's).  Returns
     `S_t * silu(g_t)` [T, W]; the state rows are advanced in place.  `max_rows`: the most rows a
     request brings, if the host knows (long portions then run chunk by chunk in parallel)."""
     _need_cuda(zxg, bias_z, bias_x, state, cu_seqlens, slots)
-    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("state", state), ("cu_seqlens", cu_seqlens), ("slots", slots)):
+    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("cu_seqlens", cu_seqlens), ("slots", slots)):
         _need_contiguous(name, t)
     _need_int32("cu_seqlens", cu_seqlens)
     _need_int32("slots", slots)
@@ -1182,8 +1182,8 @@ def gated_scan(
     requests = slots.numel()
     if cu_seqlens.numel() != requests + 1 or bias_z.numel() != width or bias_x.numel() != width:
         raise KernelShapeError("gated_scan: one more boundary than requests, one bias per column")
-    if state.dim() != 2 or state.shape[1] != width or state.shape[0] < 2:
-        raise KernelShapeError(f"gated_scan: state is [slots + 1, {width}], got {tuple(state.shape)}")
+    if state.dim() != 2 or state.shape[1] != width or state.shape[0] < 2 or state.stride(1) != 1:
+        raise KernelShapeError(f"gated_scan: state is [slots + 1, {width}] with unit inner stride, got {tuple(state.shape)}")
     out = torch.empty((tokens, width), dtype=zxg.dtype, device=zxg.device)
     chunk = chunks = 0
     summaries = None
@@ -1192,7 +1192,7 @@ def gated_scan(
         summaries = torch.empty((requests, chunks, 2, width), dtype=torch.float32, device=zxg.device)
     library.check(
         library.load().mi_gated_scan(
-            _dtype_code(zxg), _ptr(zxg), zxg.stride(0), _ptr(bias_z), _ptr(bias_x), _ptr(state), _ptr(cu_seqlens),
+            _dtype_code(zxg), _ptr(zxg), zxg.stride(0), _ptr(bias_z), _ptr(bias_x), _ptr(state), state.stride(0), _ptr(cu_seqlens),
             _ptr(slots), _ptr(out), out.stride(0), requests, width, state.shape[0] - 1, chunk, chunks, _ptr(summaries),
             _stream(),
         )

@@ -115,7 +115,10 @@ def test_gated_recurrence_over_unequal_requests_with_carried_state(dtype, length
     state = rng.standard_normal((slots + 1, width)).astype(np.float32)
     owners = [3, 0, -1, 5][: len(lengths)]
     cu = np.concatenate([[0], np.cumsum(lengths)])
-    state_d = dev(state)
+    # (state rows of different slots lie further apart than their own width, as in the engine's state buffer)
+    buffer = torch.full((slots + 1, width + 26), 9.0, device=DEV)
+    state_d = buffer[:, 3 : 3 + width]
+    state_d.copy_(dev(state))
     got = ops.gated_scan(dev(zxg, TORCH[dtype]), dev(bz), dev(bx), state_d, dev(cu, torch.int32), dev(np.array(owners), torch.int32),
                          max_rows).float().cpu().numpy()
     after = state_d.cpu().numpy()
@@ -131,6 +134,7 @@ def test_gated_recurrence_over_unequal_requests_with_carried_state(dtype, length
         assert np.abs(after[row] - last).max() < 1e-5
     for row in set(range(slots + 1)) - touched:
         assert np.array_equal(after[row], state[row])
+    assert bool((buffer[:, :3] == 9.0).all()) and bool((buffer[:, 3 + width :] == 9.0).all())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
