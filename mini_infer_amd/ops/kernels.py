@@ -1156,7 +1156,7 @@ def cast_rows(residual: torch.Tensor) -> torch.Tensor:
     return out
 
 
-GATED_SCAN_CHUNK = 32  # rows of a chunk of the chunked recurrence
+GATED_SCAN_CHUNK = 32  # rows of a chunk of the chunked recurrence where the tiled kernels do not take the shapes
 GATED_SCAN_SEQUENTIAL_ROWS = 128  # portions up to this many rows are walked by one thread a column
 
 
@@ -1188,7 +1188,10 @@ def gated_scan(
     chunk = chunks = 0
     summaries = None
     if max_rows is not None and max_rows > GATED_SCAN_SEQUENTIAL_ROWS:
-        chunk, chunks = GATED_SCAN_CHUNK, -(-max_rows // GATED_SCAN_CHUNK)
+        chunk = GATED_SCAN_CHUNK
+        if width % 8 == 0 and zxg.stride(0) % 8 == 0:  # what the tiled kernels take: their chunk is theirs to say
+            chunk = library.load().mi_gated_scan_tile_rows(_dtype_code(zxg))
+        chunks = -(-max_rows // chunk)
         summaries = torch.empty((requests, chunks, 2, width), dtype=torch.float32, device=zxg.device)
     library.check(
         library.load().mi_gated_scan(

@@ -101,14 +101,16 @@ def test_norm_on_a_sublayers_output_adds_into_the_stream(dtype, with_gain, with_
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("lengths, max_rows", [((1, 1, 1), 1), ((5, 0, 17, 2), 17), ((300, 131, 64, 1), 300), ((129,), None)])
-def test_gated_recurrence_over_unequal_requests_with_carried_state(dtype, lengths, max_rows):
+@pytest.mark.parametrize("width", [70, 72, 192])  # (columns in fours and whole tiles of 64, or neither)
+@pytest.mark.parametrize("lengths, max_rows", [((1, 1, 1), 1), ((5, 0, 17, 2), 17), ((300, 131, 64, 1), 300), ((129,), None),
+                                               ((129, 0, 200), 200)])
+def test_gated_recurrence_over_unequal_requests_with_carried_state(dtype, lengths, max_rows, width):
     """Rows of several requests in one launch, one of them without rows, one whose slot is nobody's;
     the state that comes in is not zero, and what goes out is what the next portion starts from."""
     from mini_infer_amd import ops
 
     rng = np.random.default_rng(sum(lengths))
-    width, slots = 70, 6
+    slots = 6
     total = sum(lengths)
     zxg = rounded(2.0 * rng.standard_normal((total, 3 * width)).astype(np.float32), dtype)
     bz, bx = rng.standard_normal(width).astype(np.float32), rng.standard_normal(width).astype(np.float32)
