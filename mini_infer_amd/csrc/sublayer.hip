@@ -68,7 +68,12 @@ __device__ __forceinline__ A block_total(A v, A* scratch) {
 
 __device__ __forceinline__ float inv_root(float mean_sq, float eps) { return 1.0f / sqrtf(mean_sq + eps); }
 __device__ __forceinline__ double inv_root(double mean_sq, double eps) { return 1.0 / sqrt(mean_sq + eps); }
-__device__ __forceinline__ float logistic(float z) { return 1.0f / (1.0f + expf(-z)); }
+// float32: the hardware's exponential and reciprocal (v_exp_f32, v_rcp_f32: one ulp each).  The
+// library's expf and an IEEE division cost some 70 instructions per gate, and a prompt's
+// recurrence was bound by them, not by memory (2,048 x 4,096 gates: 17 us of arithmetic).
+__device__ __forceinline__ float logistic(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.4426950408889634f));
+}
 __device__ __forceinline__ double logistic(double z) { return 1.0 / (1.0 + exp(-z)); }
 __device__ __forceinline__ float tanh_of(float z) { return tanhf(z); }
 __device__ __forceinline__ double tanh_of(double z) { return tanh(z); }
@@ -385,7 +390,9 @@ __global__ __launch_bounds__(64) void gated_scan_outputs_kernel(
 // chunk (ROWS rows).  All threads load the chunk's [z | x | g] in whole 128-byte pieces and
 // evaluate the gates of their elements at once (the exponentials are the arithmetic of this
 // kernel); keep and add go to LDS, where one wave, a lane a column, walks the rows; then all
-// threads multiply the states with silu(g), which they kept in registers, and store.  A thread
+// threads multiply the states with silu(g), which they kept in registers, and store.  There is
+// no launch between the two passes: a block of pass 3 composes the (P, Q) of the chunks before
+// its own by itself (at most a few dozen steps on values that lie in the L2).  A thread
 // that walked a column of a chunk by itself had at most 24 loads of 8 bytes in flight and
 // the kernel ran at 0.7-1.2 TB/s.
 constexpr int TILE_COLS = 64;
@@ -395,7 +402,8 @@ template <typename T, int ROWS, bool SUMMARY>
 __global__ __launch_bounds__(256) void gated_scan_tile_kernel(
     const T* __restrict__ zxg, int64_t in_stride, const float* __restrict__ bz, const float* __restrict__ bx,
     const int* __restrict__ cu, float* __restrict__ summaries, T* __restrict__ out, int64_t out_stride, int width,
-    int chunks_per_request) {
+    int chunks_per_request, float* __restrict__ state, int64_t state_stride, const int* __restrict__ slots,
+    int num_slots) {
   using A = typename Wide<T>::type;
   constexpr int PER_THREAD = ROWS / 16;  // rows of a thread: r0, r0 + 16, ...
   __shared__ A keep_s[ROWS][TILE_COLS + TILE_PAD];
@@ -433,9 +441,14 @@ __global__ __launch_bounds__(256) void gated_scan_tile_kernel(
     }
   }
   __syncthreads();
-  float* at = summaries + (((int64_t)b * chunks_per_request + k) * 2) * width;
+  // summaries of request b: entries 0..chunks-1 hold (P, Q) of its chunks, entry `chunks_per_request`
+  // holds the state the request came with (copied by pass 1, so that no block of pass 3, where
+  // the last chunk's block writes the new state, reads a state row)
+  float* mine_s = summaries + ((int64_t)b * (chunks_per_request + 1) * 2) * width;
   if (threadIdx.x < TILE_COLS && c0 + (int)threadIdx.x < width) {
     const int col = threadIdx.x;
+    const int slot = slots[b];
+    float* row = state + ((slot < 0 || slot >= num_slots) ? num_slots : slot) * state_stride + c0 + col;
     if constexpr (SUMMARY) {
       A p = 1, q = 0;
 #pragma unroll 8
@@ -444,15 +457,23 @@ __global__ __launch_bounds__(256) void gated_scan_tile_kernel(
         p *= keep;
         q = keep * q + add_s[r][col];
       }
+      float* at = mine_s + (int64_t)k * 2 * width;
       at[c0 + col] = (float)p;
       at[width + c0 + col] = (float)q;
+      if (k == 0) mine_s[(int64_t)chunks_per_request * 2 * width + c0 + col] = *row;
     } else {
-      A s = (A)at[width + c0 + col];  // the chunk's incoming state, left by pass 2
+      A s = (A)mine_s[(int64_t)chunks_per_request * 2 * width + c0 + col];
+#pragma unroll 8
+      for (int j = 0; j < k; ++j) {  // through the chunks before this one
+        const float* at = mine_s + (int64_t)j * 2 * width;
+        s = (A)at[c0 + col] * s + (A)at[width + c0 + col];
+      }
 #pragma unroll 8
       for (int r = 0; r < rows; ++r) {
         s = keep_s[r][col] * s + add_s[r][col];
         add_s[r][col] = s;
       }
+      if (first + rows == cu[b + 1]) *row = (float)s;  // the request's last chunk of this step
     }
   }
   if constexpr (!SUMMARY) {
@@ -483,13 +504,12 @@ static int gated_scan_tiles_launch(const void* zxg, int64_t in_stride, const flo
   constexpr int ROWS = tile_rows<T>();
   dim3 grid(ceil_div(width, TILE_COLS), chunks_per_request, num_requests);
   gated_scan_tile_kernel<T, ROWS, true><<<grid, 256, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, nullptr,
-                                                                  0, width, chunks_per_request);
+                                                                  0, width, chunks_per_request, state, state_stride, slots,
+                                                                  num_slots);
   MI_CHECK_LAUNCH("gated_scan (tile summaries)");
-  gated_scan_carry_kernel<<<dim3(ceil_div(width, 64), num_requests), 64, 0, stream>>>(
-      summaries, state, state_stride, cu, slots, width, ROWS, chunks_per_request, num_slots);
-  MI_CHECK_LAUNCH("gated_scan (carry)");
   gated_scan_tile_kernel<T, ROWS, false><<<grid, 256, 0, stream>>>((const T*)zxg, in_stride, bz, bx, cu, summaries, (T*)out,
-                                                                   out_stride, width, chunks_per_request);
+                                                                   out_stride, width, chunks_per_request, state,
+                                                                   state_stride, slots, num_slots);
   MI_CHECK_LAUNCH("gated_scan (tile outputs)");
   return MI_OK;
 }
@@ -524,7 +544,7 @@ static int gated_scan_launch(const void* zxg, int64_t in_stride, const float* bz
 
 // `chunk` = 0: the sequential form.  `chunk` > 0: the chunked form; no request may bring more
 // than chunk * chunks_per_request rows (the caller's bound), and `summaries` holds
-// num_requests * chunks_per_request * 2 * width floats.  `state_stride`: floats between the
+// num_requests * (chunks_per_request + 1) * 2 * width floats.  `state_stride`: floats between the
 // state rows of two slots.
 extern "C" int mi_gated_scan(int dtype, const void* zxg, int64_t in_stride, const float* bz, const float* bx,
                              float* state, int64_t state_stride, const int* cu, const int* slots, void* out,

@@ -1192,7 +1192,7 @@ def gated_scan(
         if width % 8 == 0 and zxg.stride(0) % 8 == 0:  # what the tiled kernels take: their chunk is theirs to say
             chunk = library.load().mi_gated_scan_tile_rows(_dtype_code(zxg))
         chunks = -(-max_rows // chunk)
-        summaries = torch.empty((requests, chunks, 2, width), dtype=torch.float32, device=zxg.device)
+        summaries = torch.empty((requests, chunks + 1, 2, width), dtype=torch.float32, device=zxg.device)
     library.check(
         library.load().mi_gated_scan(
             _dtype_code(zxg), _ptr(zxg), zxg.stride(0), _ptr(bias_z), _ptr(bias_x), _ptr(state), state.stride(0), _ptr(cu_seqlens),
