@@ -42,6 +42,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              way like every product of this path, so that a position's logits are the same
 //              numbers whether its step had few rows (this kernel) or many (the vendor
 //              library's bfloat16 product, widened afterwards).
+//   EPI_GELU_TABLE  c = bf16(gelu_tanh(bf16(product)) * table[ids[row], col0 + feature]): a gate that
+//              multiplies a slice of a per-token table row (a side input that depends on the
+//              token's identity); the values are those of the product followed by gated_table_rows.
 //   EPI_GATED  W holds two stacked matrices [gate; up] of n rows each and the output is
 //              silu(gate . a) * (up . a): a block computes both halves of its features,
 //              so the [m, 2n] intermediate is never written.
@@ -60,7 +63,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              The norm's launch between two products is saved.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
-enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
@@ -91,6 +94,11 @@ struct FoldArgs {  // what the folded neighbours of a product need
   int64_t ld_residual;
   const bf16_t* norm_weight;
   float* sumsq_out;
+  // EPI_GELU_TABLE: the table [rows][ld_table], the table row of each activation row, the first column
+  const bf16_t* table;
+  int64_t ld_table;
+  const int* table_ids;
+  int table_col;
   // PRO_SCALED: the pieces of the rows' sums of squares [pieces][m], the norm's eps and width
   const float* sumsq_in;
   int sumsq_pieces;
@@ -489,6 +497,19 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
         if (feature + r < n_end) dst32[r] = (float)(bf16_t)sum[r];
       continue;
     }
+    if constexpr (EPI == EPI_GELU_TABLE) {
+      const bf16_t* slice = fold.table + (int64_t)fold.table_ids[token] * fold.ld_table + fold.table_col + feature;
+      bf16_t* gated = c + (int64_t)token * ldc + feature;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (feature + r < n_end) {
+          const float z = (float)(bf16_t)sum[r];
+          const float act = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+          gated[r] = (bf16_t)(act * (float)slice[r]);
+        }
+      }
+      continue;
+    }
     bf16_t* dst = c + (int64_t)token * ldc + feature;
     if (feature + 3 < n_end && (ldc % 4 == 0)) {
       bf16x4_t packed;
@@ -567,9 +588,9 @@ static bool whole_lines(const void* w, int64_t ldw, int64_t rows, int k) {
          rows * ldw * 2 < ((int64_t)1 << 32);
 }
 
-// `out_f32`: c is float32 [m, ldc] (EPI_STORE_F32).
+// `epi`: EPI_STORE, EPI_STORE_F32 (c is float32 [m, ldc]) or EPI_GELU_TABLE (with its fields of `fold`).
 static int skinny_plain(const void* a, int64_t lda, const void* w, int64_t ldw, void* c, int64_t ldc, int m, int n,
-                        int k, bool out_f32, hipStream_t stream) {
+                        int k, int epi, hipStream_t stream, const FoldArgs nothing_folded = {}) {
   MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
              "gemm_skinny_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
@@ -577,7 +598,6 @@ static int skinny_plain(const void* a, int64_t lda, const void* w, int64_t ldw, 
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)c;
-  const FoldArgs nothing_folded = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 4);
@@ -589,8 +609,9 @@ static int skinny_plain(const void* a, int64_t lda, const void* w, int64_t ldw, 
     gemm_skinny_bf16_kernel<NT_, U_, EPI_, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded); \
   else                                                                                                             \
     gemm_skinny_bf16_kernel<NT_, U_, EPI_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldc, m, n, k, fpb, nothing_folded)
-#define SK_PLAIN(NT_, U_)                                \
-  if (out_f32) { SK_PLAIN_AS(NT_, U_, EPI_STORE_F32); } \
+#define SK_PLAIN(NT_, U_)                                                \
+  if (epi == EPI_STORE_F32) { SK_PLAIN_AS(NT_, U_, EPI_STORE_F32); }       \
+  else if (epi == EPI_GELU_TABLE) { SK_PLAIN_AS(NT_, U_, EPI_GELU_TABLE); } \
   else { SK_PLAIN_AS(NT_, U_, EPI_STORE); }
   switch (ceil_div(fpb, 16)) {
     case 1: SK_PLAIN(1, 8); break;
@@ -606,13 +627,27 @@ static int skinny_plain(const void* a, int64_t lda, const void* w, int64_t ldw, 
 
 extern "C" int mi_gemm_skinny_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* c,
                                    int64_t ldc, int m, int n, int k, hipStream_t stream) {
-  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, false, stream);
+  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, EPI_STORE, stream);
 }
 
 // The same product, the same values, written as float32 [m, ldc].
 extern "C" int mi_gemm_skinny_f32out_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, float* c,
                                           int64_t ldc, int m, int n, int k, hipStream_t stream) {
-  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, true, stream);
+  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, EPI_STORE_F32, stream);
+}
+
+// c[m, n] = gelu_tanh(a . w^T) * table[ids[row], col0 : col0 + n], bfloat16 (EPI_GELU_TABLE).
+extern "C" int mi_gemm_skinny_gelu_table_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, const void* table,
+                                              int64_t ld_table, const int* ids, int col0, int table_rows, void* c,
+                                              int64_t ldc, int m, int n, int k, hipStream_t stream) {
+  MI_REQUIRE(table != nullptr && ids != nullptr && col0 >= 0 && table_rows > 0 && ld_table >= (int64_t)col0 + n,
+             "gemm_skinny_gelu_table_bf16: columns %d..%d of a table row of %lld", col0, col0 + n, (long long)ld_table);
+  FoldArgs fold = {};
+  fold.table = (const bf16_t*)table;
+  fold.ld_table = ld_table;
+  fold.table_ids = ids;
+  fold.table_col = col0;
+  return skinny_plain(a, lda, w, ldw, c, ldc, m, n, k, EPI_GELU_TABLE, stream, fold);
 }
 
 // c[m, n] = attention output [m, heads*head_dim] . w^T, the attention output still lying in

@@ -1286,6 +1286,42 @@ def gated_table_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor,
     return out
 
 
+def linear_gelu_table(x: torch.Tensor, weight: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, first_col: int) -> torch.Tensor:
+    """`gelu_tanh(x @ weight.T) * table[ids, first_col : first_col + N]`.  Few bfloat16 rows: one
+    weight-streaming kernel with the activation and the gather in its last step; otherwise the
+    product followed by `gated_table_rows`.  Both round the product to the element type first."""
+    n = weight.shape[0]
+    if (
+        x.dtype == torch.bfloat16
+        and weight.dtype == torch.bfloat16
+        and table.dtype == torch.bfloat16
+        and x.dim() == 2
+        and weight.dim() == 2
+        and x.shape[1] == weight.shape[1]
+        and x.stride(1) == 1
+        and weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+    ):
+        _need_cuda(x, weight, table, ids)
+        _need_contiguous("table", table)
+        _need_contiguous("ids", ids)
+        _need_int32("ids", ids)
+        m, k = x.shape
+        if table.dim() != 2 or ids.numel() != m or first_col < 0 or first_col + n > table.shape[1]:
+            raise KernelShapeError(
+                f"linear_gelu_table: columns {first_col}..{first_col + n} of a table with {table.shape[1]}, {ids.numel()} ids for {m} rows"
+            )
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        library.check(
+            library.load().mi_gemm_skinny_gelu_table_bf16(
+                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(table), table.stride(0), _ptr(ids),
+                int(first_col), table.shape[0], _ptr(out), out.stride(0), m, n, k, _stream(),
+            )
+        )
+        return out
+    return gated_table_rows(linear(x, weight), table, ids, first_col)
+
+
 def sample(
     logits: torch.Tensor,
     temperature: torch.Tensor,

@@ -157,7 +157,9 @@ class TokenSideInput(FeedForward):
         assert self.table.tensor is not None, "side input used before its table was loaded"
         if isinstance(x, ops.ScaledRows):
             x = x.finish()
-        gated = ops.gated_table_rows(self.gate.forward(x), self.table.tensor, ctx.token_ids, self.first_col)
+        assert self.gate.weight is not None
+        # (few rows: the gate product, its activation and the gather are one kernel)
+        gated = ops.linear_gelu_table(x, self.gate.weight, self.table.tensor, ctx.token_ids, self.first_col)
         return self.proj.forward(gated)
 
 

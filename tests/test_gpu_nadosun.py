@@ -200,6 +200,26 @@ def test_gated_rows_of_a_shared_table(dtype):
     assert np.abs(got - want).max() < tolerance(dtype, np.abs(want).max())
 
 
+@pytest.mark.parametrize("rows, features, k", [(1, 24, 64), (8, 26, 256), (16, 128, 96), (17, 24, 64)])
+def test_gate_product_with_activation_and_gather_in_its_last_step(rows, features, k):
+    """Few bfloat16 rows run as one kernel; its values are those of the product followed by the
+    activation kernel, bit for bit (17 rows: the two-kernel route itself)."""
+    from mini_infer_amd import ops
+
+    rng = np.random.default_rng(rows + features)
+    x = tn.bf16_round(rng.standard_normal((rows, k)).astype(np.float32))
+    weight = tn.bf16_round((rng.standard_normal((features, k)) / np.sqrt(k)).astype(np.float32) * 2)
+    table = tn.bf16_round(rng.standard_normal((21, 3 * features + 5)).astype(np.float32))
+    ids = rng.integers(0, 21, size=rows)
+    args = (dev(x, torch.bfloat16), dev(weight, torch.bfloat16), dev(table, torch.bfloat16), dev(ids, torch.int32))
+    got = ops.linear_gelu_table(*args, features + 3)
+    two = ops.gated_table_rows(ops.linear(args[0], args[1]), args[2], args[3], features + 3)
+    assert torch.equal(got, two)
+    gate = tn.bf16_round((x.astype(np.float64) @ weight.astype(np.float64).T).astype(np.float32)).astype(np.float64)
+    want = pn.gelu_tanh(gate) * table[ids, features + 3 : 2 * features + 3]
+    assert np.abs(got.float().cpu().numpy() - want).max() < tolerance("bfloat16", max(1.0, np.abs(want).max()))
+
+
 # ---------------------------------------------------------------------------------------------
 # whole models under schedules
 # ---------------------------------------------------------------------------------------------
