@@ -166,7 +166,7 @@ def logits(cfg, w, tokens, store=_same, cuts=None, streams=None):
             r, carries[layer] = layer_forward(r, ids, cfg, w, layer, carries[layer], store)
             per_layer[layer].append(r)
         final = store(rms(r, eps) * float(w["final.norm"]))
-        out.append(final @ w["head"].astype(np.float64).T)
+        out.append(store(final @ w["head"].astype(np.float64).T))  # (the bfloat16 engine's head rounds its product too)
         at += n
     if streams is not None:
         streams.extend(np.concatenate(rows) for rows in per_layer)
