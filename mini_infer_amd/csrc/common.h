@@ -111,6 +111,15 @@ __device__ __forceinline__ void load_line_pair(const void* matrix, int64_t first
   upper_rows = __builtin_nontemporal_load((global_chunk*)(base + upper_at));
 }
 
+// 1 / (1 + exp(-z)) in float32 on the hardware's exponential and reciprocal (v_exp_f32, v_rcp_f32:
+// one ulp each).  The library's expf and an IEEE division cost some 70 instructions per gate,
+// and a prompt's gated recurrence was bound by them, not by memory (2,048 x 4,096 gates: 17 us
+// of arithmetic).  Every kernel that evaluates a gate of the recurrence uses this one function,
+// so a token's state does not depend on which kernel its step ran.
+__device__ __forceinline__ float mi_logistic(float z) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.4426950408889634f));
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int off = MI_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, MI_WAVE));

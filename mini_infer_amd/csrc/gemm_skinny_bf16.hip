@@ -45,6 +45,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //   EPI_GELU_TABLE  c = bf16(gelu_tanh(bf16(product)) * table[ids[row], col0 + feature]): a gate that
 //              multiplies a slice of a per-token table row (a side input that depends on the
 //              token's identity); the values are those of the product followed by gated_table_rows.
+//   EPI_GRU    W holds three stacked matrices [z; x; g] of n rows each, every row of `a` is the ONE
+//              token its request brings to the step, and the output is a step of the gated
+//              recurrence: S = (1 - sig(z + bz)) S + sig(z + bz) cand(x + bx), out = S silu(g),
+//              with S read from and written to the request's float32 state row (the values
+//              of the product followed by the recurrence kernel, bit for bit).
 //   EPI_GATED  W holds two stacked matrices [gate; up] of n rows each and the output is
 //              silu(gate . a) * (up . a): a block computes both halves of its features,
 //              so the [m, 2n] intermediate is never written.
@@ -63,7 +68,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              The norm's launch between two products is saved.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
-enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5, EPI_GRU = 6 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
@@ -94,6 +99,14 @@ struct FoldArgs {  // what the folded neighbours of a product need
   int64_t ld_residual;
   const bf16_t* norm_weight;
   float* sumsq_out;
+  // EPI_GRU: state rows [slots + 1][stride] (a slot outside 0..num_slots-1 means the spare row at
+  // num_slots), the slot of each activation row, the two gate biases [n]
+  float* gru_state;
+  int64_t gru_state_stride;
+  const int* gru_slots;
+  int gru_num_slots;
+  const float* gru_bz;
+  const float* gru_bx;
   // EPI_GELU_TABLE: the table [rows][ld_table], the table row of each activation row, the first column
   const bf16_t* table;
   int64_t ld_table;
@@ -118,7 +131,8 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
   static_assert(!LINES || U % 2 == 0, "whole lines are read for pairs of k-steps");
   // RT = tiles of 16 ROWS (tokens): a weight operand once in registers is used for every row tile
   static_assert(RT == 1 || (PRO == PRO_NONE && !ADDNORM), "more than 16 rows: plain activations, no folded norm");
-  constexpr int WT = (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
+  constexpr bool GRU = EPI == EPI_GRU;
+  constexpr int WT = GRU ? 3 * NT : (GATED || ROPE) ? 2 * NT : NT;  // weight tiles per block
   __shared__ float red[SK_WAVES][WT][256];
 
   // (with LINES made uniform for the compiler: the wave's range of K and with it the loop and
@@ -393,11 +407,37 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) sum[r] += red[wv][nt][(fq * 4 + r) * 16 + token_in_tile];
     float up[4] = {0.f, 0.f, 0.f, 0.f};  // the twin tile's sums: the up half (gated), the partner dims (rotary)
-    if (GATED || ROPE) {
+    if (GATED || ROPE || GRU) {
 #pragma unroll
       for (int wv = 0; wv < SK_WAVES; ++wv)
 #pragma unroll
         for (int r = 0; r < 4; ++r) up[r] += red[wv][NT + nt][(fq * 4 + r) * 16 + token_in_tile];
+    }
+    if constexpr (GRU) {
+      float gate[4] = {0.f, 0.f, 0.f, 0.f};  // the third stacked matrix's sums
+#pragma unroll
+      for (int wv = 0; wv < SK_WAVES; ++wv)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) gate[r] += red[wv][2 * NT + nt][(fq * 4 + r) * 16 + token_in_tile];
+      const int feature = n0 + nt * 16 + fq * 4;
+      const int slot = fold.gru_slots[token];
+      float* state = fold.gru_state +
+                     (int64_t)((slot < 0 || slot >= fold.gru_num_slots) ? fold.gru_num_slots : slot) * fold.gru_state_stride;
+      bf16_t* dst = c + (int64_t)token * ldc + feature;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (feature + r < n_end) {  // (rows past n_end repeat the last feature: its state is advanced once)
+          const float z = mi_logistic((float)(bf16_t)sum[r] + fold.gru_bz[feature + r]);
+          const float u = (float)(bf16_t)up[r] + fold.gru_bx[feature + r];
+          const float cand = u >= 0.f ? u + 0.5f : mi_logistic(u);
+          const float g = (float)(bf16_t)gate[r];
+          const float keep = 1.f - z, add = z * cand;
+          const float s = __builtin_fmaf(keep, state[feature + r], add);  // (as the recurrence kernel spells it)
+          state[feature + r] = s;
+          dst[r] = (bf16_t)(s * (g * mi_logistic(g)));
+        }
+      }
+      continue;
     }
     if constexpr (SCALED) {
       float total = 0.f;
@@ -856,6 +896,41 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
 // w then holds the query rows alone).  Half-paired rotation over the whole head,
 // cos/sin [m, head_dim/2] float32.  With `sumsq` the rows are a norm's output but for the
 // rows' factors (PRO_SCALED, as in mi_gemm_skinny_swiglu_scaled_bf16).
+// out[m, n] = one step of the gated recurrence per row from the stacked projection [z; x; g]
+// (EPI_GRU): at most 16 rows, each the only token of its request in this step.
+extern "C" int mi_gemm_skinny_gru_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, const float* bz,
+                                       const float* bx, float* state, int64_t state_stride, const int* slots,
+                                       int num_slots, void* out, int64_t ldo, int m, int n, int k, hipStream_t stream) {
+  MI_REQUIRE(mi_gemm_skinny_bf16_supported(m, n, k, lda, ldw),
+             "gemm_skinny_gru_bf16: takes 1 <= m <= 16, k a multiple of 32, rows aligned to 16 bytes; "
+             "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
+  MI_REQUIRE(lda >= k && ldw >= k && ldo >= n && state_stride >= n && num_slots >= 0 && bz && bx && state && slots,
+             "gemm_skinny_gru_bf16: a row stride is shorter than its row, or an argument is missing");
+  const bf16_t* ap = (const bf16_t*)a;
+  const bf16_t* wp = (const bf16_t*)w;
+  bf16_t* cp = (bf16_t*)out;
+  FoldArgs fold = {};
+  fold.gru_state = state;
+  fold.gru_state_stride = state_stride;
+  fold.gru_slots = slots;
+  fold.gru_num_slots = num_slots;
+  fold.gru_bz = bz;
+  fold.gru_bx = bx;
+  const int cus = compute_units();
+  MI_REQUIRE(cus > 0, "gemm_skinny_gru_bf16: cannot read the device's compute unit count");
+  const int fpb = features_per_block_for(n, cus, 1);  // one output tile = three weight tiles
+  const int blocks = ceil_div(n, fpb);
+  const int threads = 64 * SK_WAVES;
+  if (whole_lines(w, ldw, 3 * (int64_t)n, k)) {
+    gemm_skinny_bf16_kernel<1, 4, EPI_GRU, PRO_NONE, true><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k,
+                                                                                           fpb, fold);
+  } else {
+    gemm_skinny_bf16_kernel<1, 4, EPI_GRU><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, fold);
+  }
+  MI_CHECK_LAUNCH("gemm_skinny_gru_bf16");
+  return MI_OK;
+}
+
 static int rope_product(const char* name, const void* a, int64_t lda, const float* sumsq, int pieces, float eps,
                         const void* w, int64_t ldw, void* q_out, int64_t ldq, const float* cos_t,
                         const float* sin_t, const int* slot_mapping, void* k_pages, void* v_pages, int m, int k,

@@ -68,13 +68,12 @@ __device__ __forceinline__ A block_total(A v, A* scratch) {
 
 __device__ __forceinline__ float inv_root(float mean_sq, float eps) { return 1.0f / sqrtf(mean_sq + eps); }
 __device__ __forceinline__ double inv_root(double mean_sq, double eps) { return 1.0 / sqrt(mean_sq + eps); }
-// float32: the hardware's exponential and reciprocal (v_exp_f32, v_rcp_f32: one ulp each).  The
-// library's expf and an IEEE division cost some 70 instructions per gate, and a prompt's
-// recurrence was bound by them, not by memory (2,048 x 4,096 gates: 17 us of arithmetic).
-__device__ __forceinline__ float logistic(float z) {
-  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.4426950408889634f));
-}
+__device__ __forceinline__ float logistic(float z) { return mi_logistic(z); }
 __device__ __forceinline__ double logistic(double z) { return 1.0 / (1.0 + exp(-z)); }
+// keep * s + add in one rounding, spelled out: left to the compiler, two kernels that step the
+// same recurrence contracted it differently and their states differed in the last bit
+__device__ __forceinline__ float fused_step(float keep, float s, float add) { return __builtin_fmaf(keep, s, add); }
+__device__ __forceinline__ double fused_step(double keep, double s, double add) { return __builtin_fma(keep, s, add); }
 __device__ __forceinline__ float tanh_of(float z) { return tanhf(z); }
 __device__ __forceinline__ double tanh_of(double z) { return tanh(z); }
 
@@ -265,7 +264,7 @@ __device__ __forceinline__ void gru_row(const T* __restrict__ in, int width, int
   for (int k = 0; k < VEC; ++k) {
     A keep, add;
     gru_gates<A>((A)z_in[k] + bias_z[k], (A)u[k] + bias_x[k], keep, add);
-    s[k] = keep * s[k] + add;
+    s[k] = fused_step(keep, s[k], add);
     if constexpr (SUMMARY) p[k] *= keep;
     else y[k] = (float)(s[k] * ((A)g[k] * logistic((A)g[k])));
   }
@@ -455,7 +454,7 @@ __global__ __launch_bounds__(256) void gated_scan_tile_kernel(
       for (int r = 0; r < rows; ++r) {
         const A keep = keep_s[r][col];
         p *= keep;
-        q = keep * q + add_s[r][col];
+        q = fused_step(keep, q, add_s[r][col]);
       }
       float* at = mine_s + (int64_t)k * 2 * width;
       at[c0 + col] = (float)p;
@@ -470,7 +469,7 @@ __global__ __launch_bounds__(256) void gated_scan_tile_kernel(
       }
 #pragma unroll 8
       for (int r = 0; r < rows; ++r) {
-        s = keep_s[r][col] * s + add_s[r][col];
+        s = fused_step(keep_s[r][col], s, add_s[r][col]);
         add_s[r][col] = s;
       }
       if (first + rows == cu[b + 1]) *row = (float)s;  // the request's last chunk of this step

@@ -1286,6 +1286,52 @@ def gated_table_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor,
     return out
 
 
+def linear_gru_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether `linear_gru` runs these operands: at most 16 bfloat16 rows, K a multiple of 32."""
+    return (
+        x.dtype == torch.bfloat16
+        and weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and weight.dim() == 2
+        and weight.shape[0] % 3 == 0
+        and x.shape[1] == weight.shape[1]
+        and x.stride(1) == 1
+        and weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], x.shape[1], x.stride(0), weight.stride(0))
+    )
+
+
+def linear_gru(
+    x: torch.Tensor, weight: torch.Tensor, bias_z: torch.Tensor, bias_x: torch.Tensor, state: torch.Tensor, slots: torch.Tensor
+) -> torch.Tensor:
+    """The stacked projection [z; x; g] of a minGRU and ONE step of its recurrence as one kernel,
+    for a step in which every request brings exactly one token: row b of `x` belongs to the
+    request whose state row is `state[slots[b]]`.  The values are those of `linear` followed by
+    `gated_scan`, bit for bit (both round the products to bfloat16 first)."""
+    if not linear_gru_takes(x, weight):
+        raise KernelShapeError(f"linear_gru takes at most 16 bfloat16 rows and K in steps of 32; got x {tuple(x.shape)} {x.dtype}")
+    _need_cuda(x, weight, bias_z, bias_x, state, slots)
+    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("slots", slots)):
+        _need_contiguous(name, t)
+    _need_int32("slots", slots)
+    for name, t in (("bias_z", bias_z), ("bias_x", bias_x), ("state", state)):
+        _need_f32(name, t)
+    m, k = x.shape
+    n = weight.shape[0] // 3
+    if slots.numel() != m or bias_z.numel() != n or bias_x.numel() != n:
+        raise KernelShapeError("linear_gru: one slot per row, one bias per column")
+    if state.dim() != 2 or state.shape[1] != n or state.shape[0] < 2 or state.stride(1) != 1:
+        raise KernelShapeError(f"linear_gru: state is [slots + 1, {n}] with unit inner stride, got {tuple(state.shape)}")
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    library.check(
+        library.load().mi_gemm_skinny_gru_bf16(
+            _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias_z), _ptr(bias_x), _ptr(state), state.stride(0),
+            _ptr(slots), state.shape[0] - 1, _ptr(out), out.stride(0), m, n, k, _stream(),
+        )
+    )
+    return out
+
+
 def linear_gelu_table(x: torch.Tensor, weight: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, first_col: int) -> torch.Tensor:
     """`gelu_tanh(x @ weight.T) * table[ids, first_col : first_col + N]`.  Few bfloat16 rows: one
     weight-streaming kernel with the activation and the gather in its last step; otherwise the

@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -73,6 +73,7 @@ _SIGNATURES: dict[str, list] = {
     "mi_gated_scan": [c_int, _P, c_int64, _P, _P, _P, c_int64, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P, _P],
     "mi_qk_norm_kv_write": [c_int, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P],
     "mi_gated_scan_tile_rows": [c_int],
+    "mi_gemm_skinny_gru_bf16": [_P, c_int64, _P, c_int64, _P, _P, _P, c_int64, _P, c_int, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_gemm_skinny_gelu_table_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, _P, c_int, c_int, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_poly_norm": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, _P],
     "mi_gated_table_rows": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],

@@ -72,6 +72,16 @@ class MinGRU(Mixer):
             raise NotImplementedError("a recurrent mixer owns its state; it cannot read another call's")
         assert self.bias_z is not None and self.bias_x is not None, "minGRU used before its weights were loaded"
         assert isinstance(cache.state, torch.Tensor), "minGRU needs its state rows from the cache manager"
+        assert self.zxg.weight is not None
+        if (
+            ctx.host_cu_seqlens_q is not None
+            and ctx.max_q_len == 1
+            and x.shape[0] == ctx.state_slots.numel()
+            and ops.linear_gru_takes(x, self.zxg.weight)
+        ):
+            # a step of single tokens, few rows: the stacked product and the step of the recurrence are one kernel
+            gated = ops.linear_gru(x, self.zxg.weight, self.bias_z, self.bias_x, cache.state, ctx.state_slots)
+            return self.out.forward(gated)
         projected = self.zxg.forward(x)
         # (the most rows a request brings: known only where the host knows the step's boundaries)
         max_rows = ctx.max_q_len if ctx.host_cu_seqlens_q is not None else None

@@ -220,6 +220,31 @@ def test_gate_product_with_activation_and_gather_in_its_last_step(rows, features
     assert np.abs(got.float().cpu().numpy() - want).max() < tolerance("bfloat16", max(1.0, np.abs(want).max()))
 
 
+@pytest.mark.parametrize("rows, width, k", [(1, 24, 64), (8, 70, 256), (16, 256, 512), (5, 16, 32)])
+def test_stacked_product_with_one_step_of_the_recurrence_in_its_last_step(rows, width, k):
+    """Single tokens of several requests: the fused kernel leaves the outputs and the state rows that
+    the product followed by the recurrence kernel leaves, bit for bit; rows of other slots stay."""
+    from mini_infer_amd import ops
+
+    rng = np.random.default_rng(rows * width)
+    slots_n = 20
+    x = dev(tn.bf16_round(rng.standard_normal((rows, k)).astype(np.float32)), torch.bfloat16)
+    weight = dev(tn.bf16_round((2.0 * rng.standard_normal((3 * width, k)) / np.sqrt(k)).astype(np.float32)), torch.bfloat16)
+    bz, bx = dev(rng.standard_normal(width).astype(np.float32)), dev(rng.standard_normal(width).astype(np.float32))
+    start = rng.standard_normal((slots_n + 1, width + 6)).astype(np.float32)
+    owners = rng.permutation(slots_n)[:rows].astype(np.int32)
+    if rows > 1:
+        owners[1] = -1  # a padding row of a recorded step: nobody's state row
+    cu = dev(np.arange(rows + 1), torch.int32)
+    fused_buffer, plain_buffer = dev(start), dev(start)
+    fused_state, plain_state = fused_buffer[:, 2 : 2 + width], plain_buffer[:, 2 : 2 + width]
+    fused = ops.linear_gru(x, weight, bz, bx, fused_state, dev(owners, torch.int32))
+    plain = ops.gated_scan(ops.linear(x, weight), bz, bx, plain_state, cu, dev(owners, torch.int32), 1)
+    assert torch.equal(fused, plain) and torch.equal(fused_buffer, plain_buffer)
+    untouched = sorted(set(range(slots_n)) - set(int(o) for o in owners))
+    assert np.array_equal(fused_buffer.cpu().numpy()[untouched], start[untouched])
+
+
 # ---------------------------------------------------------------------------------------------
 # whole models under schedules
 # ---------------------------------------------------------------------------------------------
