@@ -89,15 +89,27 @@ __global__ __launch_bounds__(256) void embed_sinusoid_kernel(
     const double* __restrict__ freq, float* __restrict__ residual, T* __restrict__ cast, int hidden, float scale) {
   using A = typename Wide<T>::type;
   const int t = blockIdx.x;
-  const int i = blockIdx.y * blockDim.x + threadIdx.x;  // the blocks along y share a token's columns
+  // a thread takes a pair of columns (2j, 2j + 1): one angle, its sine and its cosine from one
+  // range reduction; the blocks along y share a token's pairs
+  const int j = blockIdx.y * blockDim.x + threadIdx.x;
+  const int i = 2 * j;
   if (i >= hidden) return;
-  const A angle = (A)positions[t] * (A)freq[i / 2];
-  A wave;
-  if constexpr (sizeof(T) == 4) wave = (i & 1) ? cos(angle) : sin(angle);
-  else wave = (i & 1) ? cosf(angle) : sinf(angle);
-  const float v = (float)((A)to_f32(table[(int64_t)ids[t] * hidden + i]) * (A)scale + wave);
-  residual[(int64_t)t * hidden + i] = v;
-  if (cast != nullptr) cast[(int64_t)t * hidden + i] = from_f32<T>(v);
+  const A angle = (A)positions[t] * (A)freq[j];
+  A wave[2];
+  if constexpr (sizeof(T) == 4) {
+    wave[0] = sin(angle);
+    wave[1] = cos(angle);
+  } else {
+    sincosf(angle, &wave[0], &wave[1]);
+  }
+  const T* row = table + (int64_t)ids[t] * hidden;
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    if (i + k >= hidden) break;  // (an odd width ends on a sine)
+    const float v = (float)((A)to_f32(row[i + k]) * (A)scale + wave[k]);
+    residual[(int64_t)t * hidden + i + k] = v;
+    if (cast != nullptr) cast[(int64_t)t * hidden + i + k] = from_f32<T>(v);
+  }
 }
 
 extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, const int* positions,
@@ -107,8 +119,8 @@ extern "C" int mi_embed_sinusoid(int dtype, const void* table, const int* ids, c
              num_tokens, hidden, vocab);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_sinusoid: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
-  MI_REQUIRE(ceil_div(hidden, 256) <= 65535, "embed_sinusoid: hidden=%d is too wide for one launch", hidden);
-  const dim3 grid(num_tokens, ceil_div(hidden, 256));
+  MI_REQUIRE(ceil_div(hidden, 512) <= 65535, "embed_sinusoid: hidden=%d is too wide for one launch", hidden);
+  const dim3 grid(num_tokens, ceil_div(ceil_div(hidden, 2), 256));
   if (dtype == MI_F32) {
     embed_sinusoid_kernel<float><<<grid, 256, 0, stream>>>((const float*)table, ids, positions, freq, residual,
                                                                  (float*)cast, hidden, scale);
