@@ -61,7 +61,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const int* __restrict__ token_request, const int* __restrict__ positions, T* __restrict__ out,
     int64_t out_row_stride, float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads,
     int kv_heads, int head_dim, int page_size, float scale, int window, int num_splits,
-    const float* __restrict__ slopes) {
+    const float* __restrict__ slopes, int v_dim, int64_t v_row_stride, int has_sink, float sink_logit) {
   using S = typename SumType<T>::type;
   extern __shared__ __align__(8) unsigned char q_lds_bytes[];
   S* q_lds = reinterpret_cast<S*>(q_lds_bytes);  // [GT][head_dim], pre-multiplied by the scale
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 #pragma unroll
     for (int v = 0; v < VPL; ++v) acc[g][v] = 0;
   }
-  const bool owns_dims = lane * VPL < head_dim;
+  const bool owns_dims = lane * VPL < v_dim;
   float slope[GT];
 #pragma unroll
   for (int g = 0; g < GT; ++g) slope[g] = (slopes != nullptr && g < nh) ? slopes[head0 + g] : 0.f;
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 #pragma unroll
       for (int v = 0; v < VPL; ++v) vv[v] = 0.f;
       if (owns_dims) {
-        const T* v_row = v_pages + (int64_t)rj * head_dim + lane * VPL;
+        const T* v_row = v_pages + (int64_t)rj * v_row_stride + lane * VPL;
         if constexpr (VEC || VPL <= 2) {  // (an even head size: a pair never straddles the row's end)
           const Pack<T, VPL> pk = *reinterpret_cast<const Pack<T, VPL>*>(v_row);
 #pragma unroll
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
         } else {
 #pragma unroll
           for (int v = 0; v < VPL; v += 2) {
-            if (lane * VPL + v < head_dim) {
+            if (lane * VPL + v < v_dim) {
               const Pack<T, 2> pk = *reinterpret_cast<const Pack<T, 2>*>(v_row + v);
               vv[v] = to_f32(pk.v[0]);
               vv[v + 1] = to_f32(pk.v[1]);
@@ -216,11 +216,13 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
 #pragma unroll
       for (int g = 0; g < GT; ++g) {
         if (g < nh) {
-          T* o = out + (int64_t)t * out_row_stride + (int64_t)(head0 + g) * head_dim + lane * VPL;
-          const S inv = (S)1 / l[g];
+          T* o = out + (int64_t)t * out_row_stride + (int64_t)(head0 + g) * v_dim + lane * VPL;
+          // a sink: one more term in the denominator, exp(sink_logit) on the scores' own scale
+          const S sunk = has_sink ? (S)exp((double)sink_logit - (double)m[g]) : (S)0;
+          const S inv = (S)1 / (l[g] + sunk);
 #pragma unroll
           for (int v = 0; v < VPL; ++v)
-            if (VEC || lane * VPL + v < head_dim) o[v] = from_f32<T>((float)(acc[g][v] * inv));
+            if (VEC || lane * VPL + v < v_dim) o[v] = from_f32<T>((float)(acc[g][v] * inv));
         }
       }
     }
@@ -232,7 +234,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
         if (owns_dims) {
 #pragma unroll
           for (int v = 0; v < VPL; ++v)
-            if (VEC || lane * VPL + v < head_dim) part_acc[slot * head_dim + lane * VPL + v] = (float)acc[g][v];
+            if (VEC || lane * VPL + v < v_dim) part_acc[slot * v_dim + lane * VPL + v] = (float)acc[g][v];
         }
         if (lane == 0) {
           part_ml[slot * 2] = m[g];
@@ -250,7 +252,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict__ part_acc,
                                                          const float* __restrict__ part_ml,
                                                          T* __restrict__ out, int64_t out_row_stride,
-                                                         int q_heads, int head_dim, int num_splits) {
+                                                         int q_heads, int head_dim, int num_splits,
+                                                         int has_sink, float sink_logit) {
   using S = typename SumType<T>::type;
   const int t = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -279,6 +282,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(const float* __restrict
   const float w_s = (lane < num_splits) ? expf(m_s - m_all) : 0.f;
   S l_all = 0;
   for (int s = 0; s < num_splits; ++s) l_all += (S)__shfl(l_s, s, MI_WAVE) * (S)__shfl(w_s, s, MI_WAVE);
+  if (has_sink) l_all += (S)exp((double)sink_logit - (double)m_all);
   const S inv = (S)1 / l_all;
   // The partial accumulators are read in batches of independent loads (a load per split
   // issued one after the other's use would cost a memory latency per split) and added in
@@ -326,25 +330,30 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
                                int64_t out_row_stride, float* part_acc, float* part_ml,
                                int num_tokens, int q_heads, int kv_heads, int head_dim,
                                int page_size, float scale, int window, int num_splits,
-                               const float* slopes, hipStream_t stream) {
+                               const float* slopes, hipStream_t stream, int v_dim = 0, int64_t v_row_stride = 0,
+                               int has_sink = 0, float sink_logit = 0.f) {
+  // (values as wide as the keys and packed, no sink: what the callers that say nothing mean)
+  if (v_dim <= 0) v_dim = head_dim;
+  if (v_row_stride <= 0) v_row_stride = v_dim;
   const int group = q_heads / kv_heads;
   dim3 grid(num_tokens, kv_heads * ceil_div(group, GT), num_splits);
   const size_t lds = sizeof(typename SumType<T>::type) * GT * head_dim;
-  const bool vec = head_dim % 16 == 0;
+  const bool vec = head_dim % 16 == 0 && v_dim % 16 == 0 && v_row_stride % 16 == 0;
 #define MI_ATTN_LAUNCH(VPL, VEC)                                                                  \
   attn_generic_kernel<T, VPL, VEC><<<grid, MI_WAVE, lds, stream>>>(                               \
       (const T*)q, q_row_stride, (const T*)k_pages, (const T*)v_pages, block_table, max_blocks,   \
       token_request, positions, (T*)out, out_row_stride, part_acc, part_ml, q_heads, kv_heads,    \
-      head_dim, page_size, scale, window, num_splits, slopes)
-  if (head_dim <= 64) { if (vec) MI_ATTN_LAUNCH(1, true); else MI_ATTN_LAUNCH(1, false); }
-  else if (head_dim <= 128) { if (vec) MI_ATTN_LAUNCH(2, true); else MI_ATTN_LAUNCH(2, false); }
-  else { if (vec) MI_ATTN_LAUNCH(4, true); else MI_ATTN_LAUNCH(4, false); }
+      head_dim, page_size, scale, window, num_splits, slopes, v_dim, v_row_stride, has_sink, sink_logit)
+  if (v_dim <= 64) { if (vec) MI_ATTN_LAUNCH(1, true); else MI_ATTN_LAUNCH(1, false); }
+  else if (v_dim <= 128) { if (vec) MI_ATTN_LAUNCH(2, true); else MI_ATTN_LAUNCH(2, false); }
+  else if (v_dim <= 256) { if (vec) MI_ATTN_LAUNCH(4, true); else MI_ATTN_LAUNCH(4, false); }
+  else { if (vec) MI_ATTN_LAUNCH(8, true); else MI_ATTN_LAUNCH(8, false); }
 #undef MI_ATTN_LAUNCH
   MI_CHECK_LAUNCH("attn_generic");
   if (num_splits > 1) {
     dim3 rgrid(num_tokens, q_heads);
     attn_reduce_kernel<T><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (T*)out, out_row_stride,
-                                                         q_heads, head_dim, num_splits);
+                                                         q_heads, v_dim, num_splits, has_sink, sink_logit);
     MI_CHECK_LAUNCH("attn_reduce");
   }
   return MI_OK;
@@ -352,20 +361,22 @@ static int attn_generic_launch(const void* q, int64_t q_row_stride, const void* 
 
 static int attn_generic_check(int dtype, int64_t q_row_stride, int max_blocks, int64_t out_row_stride,
                               int num_tokens, int q_heads, int kv_heads, int head_dim, int page_size,
-                              int num_pages, int window, int num_splits) {
+                              int num_pages, int window, int num_splits, int v_dim = 0, int max_head_dim = 256) {
+  if (v_dim <= 0) v_dim = head_dim;
   MI_REQUIRE(num_tokens >= 0 && q_heads > 0 && kv_heads > 0, "attn_generic: bad sizes tokens=%d q_heads=%d kv_heads=%d",
              num_tokens, q_heads, kv_heads);
   MI_REQUIRE(q_heads % kv_heads == 0, "attn_generic: q_heads=%d is not a multiple of kv_heads=%d",
              q_heads, kv_heads);
-  MI_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256,
-             "attn_generic: head_dim=%d must be even and at most 256", head_dim);
+  MI_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= max_head_dim,
+             "attn_generic: head_dim=%d must be even and at most %d", head_dim, max_head_dim);
+  MI_REQUIRE(v_dim % 2 == 0 && v_dim <= 512, "attn_generic: value rows of %d must be even and at most 512", v_dim);
   MI_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0, "attn_generic: bad page sizes page_size=%d num_pages=%d max_blocks=%d",
              page_size, num_pages, max_blocks);
   MI_REQUIRE((int64_t)num_pages * kv_heads * page_size < (int64_t)1 << 31,
              "attn_generic: the cache has too many key rows for 32-bit row indices");
   MI_REQUIRE(window >= 0, "attn_generic: window=%d must be 0 (none) or positive", window);
   MI_REQUIRE(num_splits >= 1 && num_splits <= 64, "attn_generic: num_splits=%d must be 1..64", num_splits);
-  MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * head_dim,
+  MI_REQUIRE(q_row_stride >= (int64_t)q_heads * head_dim && out_row_stride >= (int64_t)q_heads * v_dim,
              "attn_generic: row strides shorter than q_heads*head_dim");
   MI_REQUIRE(kv_heads * ceil_div(q_heads / kv_heads, GT) <= 65535, "attn_generic: too many heads");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "attn_generic: unknown dtype %d", dtype);
@@ -398,6 +409,38 @@ extern "C" int mi_attn_generic(int dtype, const void* q, int64_t q_row_stride, c
                                      num_splits, slopes, stream);
 }
 
+// The same attention with more said about it: key rows of `head_dim` and value rows of `v_dim`
+// elements that lie `v_row_stride` elements apart (a value row may be the front part of a key
+// row: pass the key pages as value pages and head_dim as the stride), key rows up to 1024 wide,
+// and optionally a sink: one more term exp(sink_logit) in the softmax's denominator that
+// carries no value.  Queries are [token][head][head_dim], outputs [token][head][v_dim];
+// part_acc holds num_tokens*q_heads*num_splits*v_dim floats.
+extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, const void* k_pages,
+                               const void* v_pages, const int* block_table, int max_blocks,
+                               const int* token_request, const int* positions, void* out,
+                               int64_t out_row_stride, float* part_acc, float* part_ml,
+                               int num_tokens, int q_heads, int kv_heads, int head_dim, int v_dim,
+                               int64_t v_row_stride, int page_size, int num_pages, float scale, int window,
+                               int num_splits, const float* slopes, int has_sink, float sink_logit,
+                               hipStream_t stream) {
+  MI_REQUIRE(v_dim > 0 && v_row_stride >= v_dim, "attn_general: value rows of %d lie %lld apart", v_dim,
+             (long long)v_row_stride);
+  const int bad = attn_generic_check(dtype, q_row_stride, max_blocks, out_row_stride, num_tokens, q_heads,
+                                     kv_heads, head_dim, page_size, num_pages, window, num_splits, v_dim, 1024);
+  if (bad != MI_OK) return bad;
+  MI_REQUIRE(num_splits == 1 || (part_acc && part_ml), "attn_general: split keys need partial buffers");
+  if (num_tokens == 0) return MI_OK;
+  if (dtype == MI_F32)
+    return attn_generic_launch<float>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                      token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                      num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                      num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit);
+  return attn_generic_launch<bf16_t>(q, q_row_stride, k_pages, v_pages, block_table, max_blocks,
+                                     token_request, positions, out, out_row_stride, part_acc, part_ml,
+                                     num_tokens, q_heads, kv_heads, head_dim, page_size, scale, window,
+                                     num_splits, slopes, stream, v_dim, v_row_stride, has_sink, sink_logit);
+}
+
 // The combining step alone, for partials written by the matrix-core kernel.
 extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
                                    int64_t out_row_stride, int num_tokens, int q_heads,
@@ -407,7 +450,7 @@ extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, 
   dim3 rgrid(num_tokens, q_heads);
   attn_reduce_kernel<bf16_t><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (bf16_t*)out,
                                                             out_row_stride, q_heads, head_dim,
-                                                            num_splits);
+                                                            num_splits, 0, 0.f);
   MI_CHECK_LAUNCH("attn_reduce");
   return MI_OK;
 }

@@ -33,12 +33,12 @@ __device__ __forceinline__ void store4(bf16_t* p, const float v[4]) {
 }
 
 // ---------------------------------------------------------------------------
-// embedding: residual[t, :] = float(table[ids[t], :])
+// embedding: residual[t, :] = float(table[ids[t], :]) * scale
 // ---------------------------------------------------------------------------
 
 template <typename T, int VEC>
 __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ residual, int hidden) {
+                                    float* __restrict__ residual, int hidden, float scale) {
   const int t = blockIdx.x;
   const T* row = table + (int64_t)ids[t] * hidden;
   float* out = residual + (int64_t)t * hidden;
@@ -46,33 +46,35 @@ __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __re
     for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
       float v[4];
       load4(row + i, v);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] *= scale;  // (times 1 changes nothing)
       store4(out + i, v);
     }
   } else {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_f32(row[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_f32(row[i]) * scale;
   }
 }
 
 template <typename T>
 static int embed_gather_launch(const void* table, const int* ids, float* residual, int num_tokens,
-                               int hidden, hipStream_t stream) {
+                               int hidden, float scale, hipStream_t stream) {
   if (num_tokens == 0) return MI_OK;
   if (hidden % 4 == 0) {
-    embed_gather_kernel<T, 4><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden);
+    embed_gather_kernel<T, 4><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden, scale);
   } else {
-    embed_gather_kernel<T, 1><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden);
+    embed_gather_kernel<T, 1><<<num_tokens, 256, 0, stream>>>((const T*)table, ids, residual, hidden, scale);
   }
   MI_CHECK_LAUNCH("embed_gather");
   return MI_OK;
 }
 
 extern "C" int mi_embed_gather(int dtype, const void* table, const int* ids, float* residual,
-                               int num_tokens, int hidden, int vocab, hipStream_t stream) {
+                               int num_tokens, int hidden, int vocab, float scale, hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && hidden > 0 && vocab > 0,
              "embed_gather: bad sizes tokens=%d hidden=%d vocab=%d", num_tokens, hidden, vocab);
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "embed_gather: unknown dtype %d", dtype);
-  if (dtype == MI_F32) return embed_gather_launch<float>(table, ids, residual, num_tokens, hidden, stream);
-  return embed_gather_launch<bf16_t>(table, ids, residual, num_tokens, hidden, stream);
+  if (dtype == MI_F32) return embed_gather_launch<float>(table, ids, residual, num_tokens, hidden, scale, stream);
+  return embed_gather_launch<bf16_t>(table, ids, residual, num_tokens, hidden, scale, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -419,7 +421,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int* __restrict__ slot_mapping, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int q_heads, int kv_heads, int head_dim, int rotary_dim,
-    int interleaved, int page_size, int v_transposed) {
+    int interleaved, int page_size, int v_transposed, int v_dim) {
   const int t = blockIdx.x;
   // the blocks along y share a token's work items
   const int first = blockIdx.y * blockDim.x + threadIdx.x;
@@ -461,11 +463,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     const int h = e / pass, d = rotary_dim + e % pass;
     k_pages[(((int64_t)page * kv_heads + h) * page_size + off) * head_dim + d] = k_row[h * head_dim + d];
   }
-  for (int e = first; e < kv_heads * head_dim; e += stride) {
-    const int h = e / head_dim, d = e % head_dim;
-    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * head_dim;
-    const int64_t at = v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * head_dim + d;
-    v_pages[at] = v_row[h * head_dim + d];
+  // (value heads are v_dim wide, which need not be the keys' width)
+  for (int e = first; e < kv_heads * v_dim; e += stride) {
+    const int h = e / v_dim, d = e % v_dim;
+    const int64_t chunk = ((int64_t)page * kv_heads + h) * page_size * v_dim;
+    const int64_t at = v_transposed ? chunk + (int64_t)d * page_size + off : chunk + (int64_t)off * v_dim + d;
+    v_pages[at] = v_row[h * v_dim + d];
   }
 }
 
@@ -586,14 +589,15 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
                                 const float* sin_t, const int* slot_mapping, void* k_pages,
                                 void* v_pages, int num_tokens, int q_heads, int kv_heads,
                                 int head_dim, int rotary_dim, int interleaved, int page_size,
-                                int num_pages, int v_transposed, hipStream_t stream) {
+                                int num_pages, int v_transposed, int v_head_dim, hipStream_t stream) {
+  if (v_head_dim <= 0) v_head_dim = head_dim;  // values as wide as keys
   MI_REQUIRE(num_tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0,
              "rope_kv_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d", num_tokens,
              q_heads, kv_heads, head_dim);
   MI_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
              "rope_kv_write: rotary_dim=%d must be even and at most head_dim=%d", rotary_dim, head_dim);
-  MI_REQUIRE(row_stride >= (int64_t)(q_heads + 2 * kv_heads) * head_dim,
-             "rope_kv_write: row stride %lld is shorter than (q+2kv)*head_dim", (long long)row_stride);
+  MI_REQUIRE(row_stride >= (int64_t)(q_heads + kv_heads) * head_dim + (int64_t)kv_heads * v_head_dim,
+             "rope_kv_write: row stride %lld is shorter than the q, k and v heads", (long long)row_stride);
   MI_REQUIRE(kv_heads == 0 || slot_mapping == nullptr || (page_size > 0 && num_pages > 0 && k_pages && v_pages),
              "rope_kv_write: pages are needed to write keys and values");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "rope_kv_write: unknown dtype %d", dtype);
@@ -602,7 +606,7 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
   const size_t elem = dtype == MI_F32 ? 4 : 2;
   const bool aligned = ((uintptr_t)qkv | (uintptr_t)cos_t | (uintptr_t)sin_t | (uintptr_t)k_pages |
                         (uintptr_t)v_pages | (uintptr_t)(row_stride * elem)) % 16 == 0;
-  if (!interleaved && aligned && head_dim % 4 == 0 && rotary_dim % 8 == 0) {
+  if (!interleaved && aligned && head_dim % 4 == 0 && rotary_dim % 8 == 0 && v_head_dim == head_dim) {
     const int items = max(q_heads * (rotary_dim / 8), kv_heads * (head_dim / 4));
     const int blocks_y = min((num_tokens >= 512) ? 2 : 16, max(1, ceil_div(items, 256)));
     dim3 grid(num_tokens, blocks_y);
@@ -619,17 +623,17 @@ extern "C" int mi_rope_kv_write(int dtype, void* qkv, int64_t row_stride, const 
     return MI_OK;
   }
   // few tokens (decode): spread each token's heads over several blocks
-  const int items = max(q_heads * (rotary_dim / 2), kv_heads * head_dim);
+  const int items = max(q_heads * (rotary_dim / 2), kv_heads * max(head_dim, v_head_dim));
   const int blocks_y = min((num_tokens >= 512) ? 4 : 16, max(1, ceil_div(items, 256)));
   dim3 grid(num_tokens, blocks_y);
   if (dtype == MI_F32) {
     rope_kv_write_kernel<float><<<grid, 256, 0, stream>>>(
         (float*)qkv, row_stride, cos_t, sin_t, slot_mapping, (float*)k_pages, (float*)v_pages,
-        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed, v_head_dim);
   } else {
     rope_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, cos_t, sin_t, slot_mapping, (bf16_t*)k_pages, (bf16_t*)v_pages,
-        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed);
+        q_heads, kv_heads, head_dim, rotary_dim, interleaved, page_size, v_transposed, v_head_dim);
   }
   MI_CHECK_LAUNCH("rope_kv_write");
   return MI_OK;

@@ -23,6 +23,18 @@ from mini_infer_amd.parts.base import (
 from mini_infer_amd.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 
 
+def _with_shift(delta, shift: torch.Tensor):
+    """`delta` (what is still to be added to the stream: nothing, a tensor, or anything with
+    `finish()`) with the float32 vector `shift` added to every row as well."""
+    from mini_infer_amd import ops
+
+    if isinstance(delta, ops.StreamUpdate):
+        return delta.shifted(shift)
+    if delta is not None and hasattr(delta, "finish"):
+        delta = delta.finish()
+    return ops.StreamUpdate(delta, shift=shift)
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device) -> None:
         import mini_infer_amd.parts  # noqa: F401  (registers the built-in part kinds)
@@ -40,6 +52,7 @@ class DecoderModel:
         self.final_norm = NORMS.lookup(spec.final_norm["kind"])(spec.final_norm, dtype, device, shared)
         head = spec.head_description()
         self.head = HEADS.lookup(head["kind"])(head, dtype, device, shared)
+        self.stream_vectors: dict[str, torch.Tensor] = {}  # float32 [rows, hidden], by checkpoint name
         # a product whose output only ever meets norms that can add up its pieces may leave them apart
         if self.final_norm.takes_partial_sums and all(block.takes_partial_sums for block in self.blocks):
             for block in self.blocks:
@@ -77,6 +90,8 @@ class DecoderModel:
             specs.update(block.param_specs(layer.prefix))
         specs.update(self.final_norm.param_specs(self.spec.final_norm_prefix))
         specs.update(self.head.param_specs(""))
+        for name, rows in self.spec.stream_vectors.items():
+            specs[name] = ParamSpec((rows, self.spec.hidden_size), dtype="float32")
         return specs
 
     def optional_names(self) -> set[str]:
@@ -88,6 +103,8 @@ class DecoderModel:
             block.load_params(layer.prefix, get)
         self.final_norm.load_params(self.spec.final_norm_prefix, get)
         self.head.load_params("", get)
+        for name in self.spec.stream_vectors:
+            self.stream_vectors[name] = get(name).float().contiguous()
 
     # -- cache ----------------------------------------------------------------
 
@@ -107,6 +124,10 @@ class DecoderModel:
         for i, call in enumerate(self.spec.order):
             own = call.reads_cache_of is None
             cache = caches[i if own else call.reads_cache_of]
+            if call.stream_add is not None:
+                # one more vector for every row, added with whatever the last block left to add
+                name, row = call.stream_add
+                delta = _with_shift(delta, self.stream_vectors[name][row])
             delta = self.blocks[call.layer].forward(delta, residual, ctx, cache, writes_cache=own)
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)

@@ -24,6 +24,10 @@ class LayerSpec:
 class LayerCall:
     layer: int  # index into ModelSpec.layers
     reads_cache_of: int | None = None  # index of an earlier call in `order`, or None for its own cache
+    # (name, row) of one of the model's `stream_vectors`: that row is added to every token's
+    # stream right before this call (a stack that runs some layers several times tells each pass
+    # which one it is this way)
+    stream_add: tuple[str, int] | None = None
 
 
 @dataclasses.dataclass(frozen=True)
@@ -50,6 +54,9 @@ class ModelSpec:
     max_position_embeddings: int | None = None
     embedding: dict[str, Any] | None = None
     head: dict[str, Any] | None = None
+    # checkpoint name -> number of rows of a float32 table [rows, hidden_size] whose rows calls add
+    # to the stream (`LayerCall.stream_add`)
+    stream_vectors: dict[str, int] = dataclasses.field(default_factory=dict)
 
     def embedding_description(self) -> dict[str, Any]:
         if self.embedding is not None:
@@ -71,6 +78,10 @@ class ModelSpec:
         for i, call in enumerate(self.order):
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"call {i} names layer {call.layer}, but there are {len(self.layers)} layers")
+            if call.stream_add is not None:
+                name, row = call.stream_add
+                if name not in self.stream_vectors or not 0 <= row < self.stream_vectors[name]:
+                    raise ValueError(f"call {i} adds row {row} of {name!r}, which the spec's stream_vectors do not hold")
             if call.reads_cache_of is not None:
                 if not 0 <= call.reads_cache_of < i:
                     raise ValueError(f"call {i} reads the cache of call {call.reads_cache_of}, which is not earlier")

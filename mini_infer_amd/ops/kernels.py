@@ -45,8 +45,9 @@ def _need_int32(name: str, t: torch.Tensor | None) -> None:
         raise KernelShapeError(f"{name} must be int32, got {t.dtype}")
 
 
-def _check_v_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: bool) -> None:
+def _check_v_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: bool, v_dim: int | None = None) -> None:
     pages, heads, page_size, head_dim = k_pages.shape
+    head_dim = head_dim if v_dim is None else v_dim  # (value rows of a width of their own)
     expected = (pages, heads, head_dim, page_size) if v_transposed else (pages, heads, page_size, head_dim)
     if tuple(v_pages.shape) != expected:
         raise KernelShapeError(
@@ -89,8 +90,8 @@ def _stream() -> int:
 # ----------------------------------------------------------------------------
 
 
-def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
-    """`float32(table[ids])`: the start of the residual stream, [T, H] float32."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """`float32(table[ids]) * scale`: the start of the residual stream, [T, H] float32."""
     _need_cuda(table, ids)
     _need_contiguous("table", table)
     _need_contiguous("ids", ids)
@@ -101,7 +102,7 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     library.check(
         lib.mi_embed_gather(
             _dtype_code(table), _ptr(table), _ptr(ids), _ptr(out), ids.numel(), hidden, vocab,
-            _stream(),
+            float(scale), _stream(),
         )
     )
     return out
@@ -261,8 +262,10 @@ def rope_kv_write(
     rotary_dim: int,
     interleaved: bool = False,
     v_transposed: bool = False,
+    v_head_dim: int | None = None,
 ) -> None:
     """Rotate q in place inside `qkv`; rotate k and write k, v into their page slots.
+    `v_head_dim`: the width of a value head where it is not the keys' (`head_dim`).
 
     `qkv` is [T, (q_heads + 2*kv_heads) * head_dim] (rows may be strided); pages are
     [num_pages, kv_heads, page_size, head_dim], value pages
@@ -279,10 +282,11 @@ def rope_kv_write(
     if qkv.dim() != 2 or qkv.stride(1) != 1:
         raise KernelShapeError(f"qkv must be [T, width] with unit inner stride, got {qkv.stride()}")
     tokens = qkv.shape[0]
-    if qkv.shape[1] < (q_heads + 2 * kv_heads) * head_dim:
+    v_dim = head_dim if v_head_dim is None else int(v_head_dim)
+    if qkv.shape[1] < (q_heads + kv_heads) * head_dim + kv_heads * v_dim:
         raise KernelShapeError(
-            f"qkv rows hold {qkv.shape[1]} values, fewer than (q+2kv)*head_dim = "
-            f"{(q_heads + 2 * kv_heads) * head_dim}"
+            f"qkv rows hold {qkv.shape[1]} values, fewer than the q, k and v heads need: "
+            f"{(q_heads + kv_heads) * head_dim + kv_heads * v_dim}"
         )
     if cos.shape != (tokens, rotary_dim // 2) or sin.shape != cos.shape or cos.dtype != torch.float32:
         raise KernelShapeError(
@@ -298,7 +302,7 @@ def rope_kv_write(
             raise KernelShapeError(
                 f"pages must be [num_pages, {kv_heads}, page_size, {head_dim}], got {tuple(k_pages.shape)}"
             )
-        _check_v_pages(k_pages, v_pages, v_transposed)
+        _check_v_pages(k_pages, v_pages, v_transposed, v_dim)
         if slot_mapping.numel() != tokens:
             raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
         num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
@@ -307,7 +311,7 @@ def rope_kv_write(
         lib.mi_rope_kv_write(
             _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
             _ptr(k_pages), _ptr(v_pages), tokens, q_heads, kv_heads, head_dim, rotary_dim,
-            int(interleaved), page_size, num_pages, int(v_transposed), _stream(),
+            int(interleaved), page_size, num_pages, int(v_transposed), v_dim, _stream(),
         )
     )
 
@@ -905,8 +909,15 @@ def paged_attention(
     force_plain: bool = False,
     combine: bool = True,
     slopes: torch.Tensor | None = None,
+    v_head_dim: int | None = None,
+    sink_logit: float | None = None,
 ) -> torch.Tensor | AttentionPieces:
     """Causal attention of every token over its request's pages; returns [T, q_heads*head_dim].
+
+    `v_head_dim`: value rows of another width than the keys' (the result is then
+    [T, q_heads*v_head_dim]); with `v_pages=None` a value row is the first `v_head_dim` entries
+    of its key row.  `sink_logit`: the softmax's denominator gets one more term
+    exp(sink_logit), a sink that carries no value.  These run the plain kernel.
 
     `slopes` (float32 [q_heads], optional): the score of head h for the key at position j
     seen from position p gets `slopes[h] * (j - p)` added before the softmax.  Only the
@@ -926,6 +937,12 @@ def paged_attention(
     bfloat16 caches with transposed values run on the matrix cores; everything else
     (float32, other head or page sizes) runs the plain kernel.
     """
+    if v_pages is None or sink_logit is not None or (v_head_dim is not None and v_head_dim != head_dim):
+        return _paged_attention_general(
+            q, k_pages, v_pages, block_table, token_request, positions, q_heads=q_heads, kv_heads=kv_heads,
+            head_dim=head_dim, v_head_dim=head_dim if v_head_dim is None else int(v_head_dim), scale=scale,
+            window=window, max_seq_len=max_seq_len, v_transposed=v_transposed, slopes=slopes, sink_logit=sink_logit,
+        )
     _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, cu_seqlens_q)
     for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
                     ("token_request", token_request), ("positions", positions),
@@ -1073,6 +1090,70 @@ def paged_attention(
             block_table.shape[1], _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0),
             _ptr(part_acc), _ptr(part_ml), tokens, q_heads, kv_heads, head_dim, page_size, num_pages,
             float(scale), int(window or 0), splits, _ptr(slopes), _stream(),
+        )
+    )
+    return out
+
+
+GENERAL_ATTENTION_MAX_KEY_DIM = 1024
+GENERAL_ATTENTION_MAX_VALUE_DIM = 512
+
+
+def _paged_attention_general(
+    q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor | None, block_table: torch.Tensor,
+    token_request: torch.Tensor, positions: torch.Tensor, *, q_heads: int, kv_heads: int, head_dim: int,
+    v_head_dim: int, scale: float, window: int | None, max_seq_len: int, v_transposed: bool,
+    slopes: torch.Tensor | None, sink_logit: float | None,
+) -> torch.Tensor:
+    """The plain attention kernel with everything it can be told: see `paged_attention`."""
+    _need_cuda(q, k_pages, v_pages, block_table, token_request, positions, slopes)
+    for name, t in (("k_pages", k_pages), ("v_pages", v_pages), ("block_table", block_table),
+                    ("token_request", token_request), ("positions", positions), ("slopes", slopes)):
+        _need_contiguous(name, t)
+    for name, t in (("block_table", block_table), ("token_request", token_request), ("positions", positions)):
+        _need_int32(name, t)
+    if v_transposed:
+        raise KernelShapeError("the plain attention kernel reads value pages that are not transposed")
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < q_heads * head_dim:
+        raise KernelShapeError(f"q must be [T, >= {q_heads * head_dim}] with unit inner stride")
+    if k_pages.dtype != q.dtype or k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != head_dim:
+        raise KernelShapeError(
+            f"key pages must be {q.dtype} [num_pages, {kv_heads}, page_size, {head_dim}], got {k_pages.dtype} {tuple(k_pages.shape)}"
+        )
+    num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+    if v_pages is None:
+        if not 0 < v_head_dim <= head_dim:
+            raise KernelShapeError(f"a value row inside a key row of {head_dim} cannot be {v_head_dim} wide")
+        values, v_row_stride = k_pages, head_dim
+    else:
+        if v_pages.dtype != q.dtype or tuple(v_pages.shape) != (num_pages, kv_heads, page_size, v_head_dim):
+            raise KernelShapeError(
+                f"value pages must be {q.dtype} {(num_pages, kv_heads, page_size, v_head_dim)}, got {v_pages.dtype} {tuple(v_pages.shape)}"
+            )
+        values, v_row_stride = v_pages, v_head_dim
+    if head_dim % 2 or v_head_dim % 2 or head_dim > GENERAL_ATTENTION_MAX_KEY_DIM or v_head_dim > GENERAL_ATTENTION_MAX_VALUE_DIM:
+        raise KernelShapeError(
+            f"the plain attention kernel takes even key rows up to {GENERAL_ATTENTION_MAX_KEY_DIM} and even value rows "
+            f"up to {GENERAL_ATTENTION_MAX_VALUE_DIM}, got {head_dim} and {v_head_dim}"
+        )
+    tokens = q.shape[0]
+    if token_request.numel() != tokens or positions.numel() != tokens or block_table.dim() != 2:
+        raise KernelShapeError("token_request and positions need one entry per token, block_table is [requests, max_blocks]")
+    if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != q_heads):
+        raise KernelShapeError(f"slopes must be float32 [{q_heads}], got {slopes.dtype} x {slopes.numel()}")
+    out = torch.empty((tokens, q_heads * v_head_dim), dtype=q.dtype, device=q.device)
+    group = q_heads // kv_heads
+    splits = attention_splits(tokens * kv_heads * math.ceil(group / 4), max_seq_len)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((tokens * q_heads * splits, v_head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * q_heads * splits, 2), dtype=torch.float32, device=q.device)
+    library.check(
+        library.load().mi_attn_general(
+            _dtype_code(q), _ptr(q), q.stride(0), _ptr(k_pages), _ptr(values), _ptr(block_table), block_table.shape[1],
+            _ptr(token_request), _ptr(positions), _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), tokens,
+            q_heads, kv_heads, head_dim, v_head_dim, v_row_stride, page_size, num_pages, float(scale), int(window or 0),
+            splits, _ptr(slopes), int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
         )
     )
     return out
@@ -1366,6 +1447,260 @@ def linear_gelu_table(x: torch.Tensor, weight: torch.Tensor, table: torch.Tensor
         )
         return out
     return gated_table_rows(linear(x, weight), table, ids, first_col)
+
+
+# ----------------------------------------------------------------------------
+# a layer whose sublayers share one norm and add their outputs together; a matrix-state
+# recurrence behind a short convolution; attention over one latent row per token
+# ----------------------------------------------------------------------------
+
+
+@dataclasses.dataclass
+class StreamUpdate:
+    """An update of the float32 stream that has not been made yet:
+
+        x += scale * (a + b + bias) + shift
+
+    `a`, `b`: a layer's sublayer outputs [T, H] in the compute dtype (either may be None);
+    `bias`, `shift`: float32 [H] or None.  A norm that knows it makes the update and its own
+    statistics in one launch (`stream_update_norm`); anything else calls `finish()`, which
+    returns the whole right-hand side as one float32 tensor to add."""
+
+    a: torch.Tensor | None
+    b: torch.Tensor | None = None
+    bias: torch.Tensor | None = None
+    shift: torch.Tensor | None = None
+    scale: float = 1.0
+
+    def shifted(self, shift: torch.Tensor) -> "StreamUpdate":
+        """The same update with one more vector added to every row."""
+        total = shift if self.shift is None else self.shift + shift
+        return dataclasses.replace(self, shift=total)
+
+    def finish(self) -> torch.Tensor:
+        total = None
+        for part in (self.a, self.b, self.bias):
+            if part is not None:
+                total = part.float() if total is None else total + part.float()
+        if total is not None:
+            total = total * self.scale
+        if self.shift is not None:
+            total = self.shift if total is None else total + self.shift
+        if total is None:
+            raise ValueError("an empty stream update")
+        return total
+
+
+def stream_update_norm(
+    update: StreamUpdate | None, residual: torch.Tensor, weight: torch.Tensor | None, eps: float,
+    rows: torch.Tensor | None = None,
+) -> torch.Tensor | None:
+    """Make `update` on the float32 stream in place (kept unless `rows`), then the RMS norm of the
+    new rows times `weight` (compute dtype) -> [T, H] or [len(rows), H]; `weight=None`: the
+    update alone."""
+    update = update if update is not None else StreamUpdate(None)
+    _need_cuda(update.a, update.b, update.bias, update.shift, residual, weight, rows)
+    for name, t in (("residual", residual), ("weight", weight), ("rows", rows), ("bias", update.bias), ("shift", update.shift)):
+        _need_contiguous(name, t)
+    _need_int32("rows", rows)
+    _need_f32("residual", residual)
+    _need_f32("bias", update.bias)
+    _need_f32("shift", update.shift)
+    tokens, hidden = residual.shape
+    dtype = weight.dtype if weight is not None else (update.a.dtype if update.a is not None else torch.float32)
+    for name, t in (("a", update.a), ("b", update.b)):
+        if t is not None and (t.dim() != 2 or tuple(t.shape) != (tokens, hidden) or t.stride(1) != 1 or t.dtype != dtype):
+            raise KernelShapeError(f"stream update: {name} {tuple(t.shape)} {t.dtype} does not fit the stream {(tokens, hidden)} in {dtype}")
+    for name, t in (("bias", update.bias), ("shift", update.shift), ("weight", weight)):
+        if t is not None and t.numel() != hidden:
+            raise KernelShapeError(f"stream update: {name} has {t.numel()} entries for {hidden} columns")
+    if weight is None and rows is not None:
+        raise KernelShapeError("stream update: a row list only goes with a norm")
+    n_out = tokens if rows is None else rows.numel()
+    out = torch.empty((n_out, hidden), dtype=dtype, device=residual.device) if weight is not None else None
+    code = F32 if dtype == torch.float32 else BF16
+    library.check(
+        library.load().mi_stream_update_norm(
+            code, _ptr(update.a), 0 if update.a is None else update.a.stride(0), _ptr(update.b),
+            0 if update.b is None else update.b.stride(0), _ptr(update.bias), _ptr(update.shift), float(update.scale),
+            _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), n_out, hidden, float(eps), _stream(),
+        )
+    )
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, bias: torch.Tensor | None, limit: float, slope: float) -> torch.Tensor:
+    """Rows [gate | up] (+ `bias`, float32 [2I]) -> `g * logistic(slope * g) * (u + 1)` with
+    g = min(gate, limit), u = clamp(up, -limit, limit); returns [T, I]."""
+    _need_cuda(gate_up, bias)
+    _need_contiguous("bias", bias)
+    _need_f32("bias", bias)
+    if gate_up.dim() != 2 or gate_up.stride(1) != 1 or gate_up.shape[1] % 2 != 0:
+        raise KernelShapeError(f"clamped_glu: rows hold [gate | up], got {tuple(gate_up.shape)} strides {gate_up.stride()}")
+    tokens, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    if bias is not None and bias.numel() != 2 * inter:
+        raise KernelShapeError(f"clamped_glu: the bias has {bias.numel()} entries for {2 * inter} columns")
+    out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+    library.check(
+        library.load().mi_clamped_glu(
+            _dtype_code(gate_up), _ptr(gate_up), gate_up.stride(0), _ptr(bias), _ptr(out), out.stride(0), tokens, inter,
+            float(limit), float(slope), _stream(),
+        )
+    )
+    return out
+
+
+def short_conv(
+    x: torch.Tensor, channels: int, taps_weight: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
+    slots: torch.Tensor, token_request: torch.Tensor,
+) -> torch.Tensor:
+    """A causal convolution over time per channel, then silu, on the first `channels` columns of
+    `x` [T, >= channels]: `y[t, c] = silu(sum_j w[c, j] * x[t - (taps-1) + j, c])` within each
+    request.  `tail` [slots + 1, taps - 1, channels] (compute dtype, rows may be strided) holds
+    each request's last taps-1 inputs and is advanced in place; `taps_weight` is float32
+    [channels, taps], last column the current token's."""
+    _need_cuda(x, taps_weight, tail, cu_seqlens, slots, token_request)
+    for name, t in (("taps_weight", taps_weight), ("cu_seqlens", cu_seqlens), ("slots", slots), ("token_request", token_request)):
+        _need_contiguous(name, t)
+    for name, t in (("cu_seqlens", cu_seqlens), ("slots", slots), ("token_request", token_request)):
+        _need_int32(name, t)
+    _need_f32("taps_weight", taps_weight)
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < channels:
+        raise KernelShapeError(f"short_conv: x must be [T, >= {channels}] with unit inner stride, got {tuple(x.shape)}")
+    if taps_weight.dim() != 2 or taps_weight.shape[0] != channels:
+        raise KernelShapeError(f"short_conv: taps are [{channels}, taps], got {tuple(taps_weight.shape)}")
+    taps = taps_weight.shape[1]
+    tokens, requests = x.shape[0], slots.numel()
+    if tail.dtype != x.dtype or tail.dim() != 3 or tuple(tail.shape[1:]) != (taps - 1, channels) or tail.shape[0] < 2:
+        raise KernelShapeError(f"short_conv: the tail is {x.dtype} [slots + 1, {taps - 1}, {channels}], got {tail.dtype} {tuple(tail.shape)}")
+    if taps > 1 and (tail.stride(2) != 1 or tail.stride(1) != channels):
+        raise KernelShapeError(f"short_conv: a slot's tail must be packed, got strides {tail.stride()}")
+    if cu_seqlens.numel() != requests + 1 or token_request.numel() != tokens:
+        raise KernelShapeError("short_conv: one more boundary than requests, one request index per token")
+    y = torch.empty((tokens, channels), dtype=x.dtype, device=x.device)
+    library.check(
+        library.load().mi_short_conv(
+            _dtype_code(x), _ptr(x), x.stride(0), _ptr(taps_weight), _ptr(tail), tail.stride(0), _ptr(cu_seqlens), _ptr(slots),
+            _ptr(token_request), _ptr(y), y.stride(0), tokens, requests, channels, taps, tail.shape[0] - 1, _stream(),
+        )
+    )
+    return y
+
+
+def delta_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int, int]:
+    """How `gated_delta` lays a request's state out: per head [ceil(dim/4)][vdim][4], element
+    (i, j) of S at [i // 4][j][i % 4]."""
+    return (heads, -(-dim // 4), vdim, 4)
+
+
+def gated_delta(
+    qkv: torch.Tensor, proj: torch.Tensor, col_b: int, col_a: int, col_g: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
+    norm_weight: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, *, heads: int,
+    kv_heads: int, dim: int, vdim: int, eps: float,
+) -> torch.Tensor:
+    """The gated delta rule over the rows of a step.  `qkv` [T, 2*kv_heads*dim + heads*vdim]: the
+    convolved q | k | v; `proj` [T, ...]: the rows that hold, from columns `col_b`, `col_a`
+    (heads each) and `col_g` (heads*vdim) on, the projections of the write gate, the decay and
+    the output gate.  `state` float32 [slots + 1, *delta_state_shape(...)] is advanced in
+    place.  Returns `rms_norm(S^T q) * norm_weight * silu(g)` [T, heads*vdim]."""
+    _need_cuda(qkv, proj, a_log, dt_bias, norm_weight, state, cu_seqlens, slots)
+    for name, t in (("a_log", a_log), ("dt_bias", dt_bias), ("norm_weight", norm_weight), ("cu_seqlens", cu_seqlens), ("slots", slots)):
+        _need_contiguous(name, t)
+    for name, t in (("a_log", a_log), ("dt_bias", dt_bias), ("norm_weight", norm_weight), ("state", state)):
+        _need_f32(name, t)
+    _need_int32("cu_seqlens", cu_seqlens)
+    _need_int32("slots", slots)
+    width = 2 * kv_heads * dim + heads * vdim
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < width:
+        raise KernelShapeError(f"gated_delta: qkv must be [T, >= {width}] with unit inner stride, got {tuple(qkv.shape)}")
+    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[0] != qkv.shape[0] or proj.dtype != qkv.dtype:
+        raise KernelShapeError("gated_delta: the gates' projections are rows of the same step and dtype")
+    if max(col_b + heads, col_a + heads, col_g + heads * vdim) > proj.shape[1]:
+        raise KernelShapeError("gated_delta: the gates' columns lie outside the projections' rows")
+    if a_log.numel() != heads or dt_bias.numel() != heads or norm_weight.numel() != vdim:
+        raise KernelShapeError("gated_delta: one decay rate and one step bias per head, one norm weight per value column")
+    shape = delta_state_shape(heads, dim, vdim)
+    if state.dim() != 5 or tuple(state.shape[1:]) != shape or state.shape[0] < 2 or not state[0].is_contiguous():
+        raise KernelShapeError(f"gated_delta: the state is float32 [slots + 1, {shape}] with packed slots, got {tuple(state.shape)}")
+    requests = slots.numel()
+    if cu_seqlens.numel() != requests + 1:
+        raise KernelShapeError("gated_delta: one more boundary than requests")
+    out = torch.empty((qkv.shape[0], heads * vdim), dtype=qkv.dtype, device=qkv.device)
+    library.check(
+        library.load().mi_gated_delta(
+            _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(col_b), int(col_a), int(col_g),
+            _ptr(a_log), _ptr(dt_bias), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(slots),
+            _ptr(out), out.stride(0), requests, heads, kv_heads, dim, vdim, float(eps), state.shape[0] - 1, _stream(),
+        )
+    )
+    return out
+
+
+def latent_prepare(
+    proj: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor, slot_mapping: torch.Tensor | None,
+    k_pages: torch.Tensor | None, queries: torch.Tensor, *, heads: int, q_head_width: int, q_rot_at: int, c_col: int,
+    rank: int, rot: int, eps: float,
+) -> None:
+    """What a latent attention layer does between its projections and its attention.  `proj`
+    [T, ...] holds the query heads (`q_head_width` columns each from column 0 on, the part to
+    rotate `rot` wide from `q_rot_at` inside a head) and from `c_col` on [x_c (rank) | x_r (rot)].
+    Writes `[rms_norm(x_c) * norm_weight | rotated x_r]` into the token's slot of `k_pages`
+    ([num_pages, 1, page_size, rank + rot]; nothing with `slot_mapping=None`) and each head's
+    rotated query part into the last `rot` columns of its [rank + rot] wide piece of `queries`."""
+    _need_cuda(proj, cos, sin, norm_weight, slot_mapping, k_pages, queries)
+    for name, t in (("cos", cos), ("sin", sin), ("norm_weight", norm_weight), ("slot_mapping", slot_mapping), ("k_pages", k_pages)):
+        _need_contiguous(name, t)
+    _need_int32("slot_mapping", slot_mapping)
+    _need_f32("norm_weight", norm_weight)
+    tokens = proj.shape[0]
+    if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < max(heads * q_head_width, c_col + rank + rot):
+        raise KernelShapeError(f"latent_prepare: the projections' rows are too short, got {tuple(proj.shape)}")
+    if queries.dtype != proj.dtype or queries.dim() != 2 or queries.stride(1) != 1 or tuple(queries.shape) != (tokens, heads * (rank + rot)):
+        raise KernelShapeError(f"latent_prepare: queries are {proj.dtype} [{tokens}, {heads * (rank + rot)}], got {queries.dtype} {tuple(queries.shape)}")
+    if cos.dtype != torch.float32 or tuple(cos.shape) != (tokens, rot // 2) or sin.shape != cos.shape or sin.dtype != torch.float32:
+        raise KernelShapeError(f"latent_prepare: cos/sin must be float32 [{tokens}, {rot // 2}], got {tuple(cos.shape)} {cos.dtype}")
+    if norm_weight.numel() != rank:
+        raise KernelShapeError(f"latent_prepare: the norm weight has {norm_weight.numel()} entries for a latent of {rank}")
+    if slot_mapping is not None:
+        if k_pages is None or k_pages.dtype != proj.dtype or k_pages.dim() != 4 or k_pages.shape[1] != 1 or k_pages.shape[3] != rank + rot:
+            raise KernelShapeError(f"latent_prepare: key pages must be {proj.dtype} [num_pages, 1, page_size, {rank + rot}]")
+        if slot_mapping.numel() != tokens:
+            raise KernelShapeError(f"slot_mapping has {slot_mapping.numel()} entries for {tokens} tokens")
+    library.check(
+        library.load().mi_latent_prepare(
+            _dtype_code(proj), _ptr(proj), proj.stride(0), 0, int(q_head_width), int(q_rot_at), int(c_col), _ptr(cos), _ptr(sin),
+            _ptr(norm_weight), _ptr(slot_mapping), _ptr(k_pages) if slot_mapping is not None else None, _ptr(queries),
+            queries.stride(0), tokens, heads, rank, rot, float(eps), _stream(),
+        )
+    )
+
+
+def linear_per_head(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+    """`out[:, h, :] = x[:, h, :] @ weight[h].T` for every head h: x [T, heads, K], weight
+    [heads, N, K], out [T, heads, N]; x and out may be views into wider rows (unit inner
+    stride).  float32: the true-float32 product, head by head; few bfloat16 rows: the
+    weight-streaming product, head by head; else one batched product of the vendor library."""
+    _need_cuda(x, weight, out)
+    if x.dim() != 3 or weight.dim() != 3 or out.dim() != 3 or x.stride(2) != 1 or out.stride(2) != 1 or weight.stride(2) != 1:
+        raise KernelShapeError("linear_per_head: x [T, heads, K], weight [heads, N, K], out [T, heads, N], unit inner strides")
+    tokens, heads, k = x.shape
+    n = weight.shape[1]
+    if tuple(weight.shape) != (heads, n, k) or tuple(out.shape) != (tokens, heads, n) or not (x.dtype == weight.dtype == out.dtype):
+        raise KernelShapeError(f"linear_per_head: shapes {tuple(x.shape)}, {tuple(weight.shape)}, {tuple(out.shape)} do not fit")
+    if tokens == 0:
+        return
+    lib = library.load()
+    if x.dtype == torch.float32:
+        for h in range(heads):
+            library.check(lib.mi_gemm_f32(_ptr(x[:, h]), x.stride(0), _ptr(weight[h]), weight.stride(1), _ptr(out[:, h]),
+                                          out.stride(0), tokens, n, k, _stream()))
+        return
+    if skinny_gemm_takes(tokens, k, x.stride(0), weight.stride(1)) and x.stride(1) % 8 == 0 and weight.stride(0) % 8 == 0:
+        for h in range(heads):
+            library.check(lib.mi_gemm_skinny_bf16(_ptr(x[:, h]), x.stride(0), _ptr(weight[h]), weight.stride(1),
+                                                  _ptr(out[:, h]), out.stride(0), tokens, n, k, _stream()))
+        return
+    torch.bmm(x.transpose(0, 1), weight.transpose(1, 2), out=out.transpose(0, 1))
 
 
 def sample(

@@ -14,21 +14,21 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
 
 _P = c_void_p
 _SIGNATURES: dict[str, list] = {
-    "mi_embed_gather": [c_int, _P, _P, _P, c_int, c_int, c_int, _P],
+    "mi_embed_gather": [c_int, _P, _P, _P, c_int, c_int, c_int, c_float, _P],
     "mi_take_device_tokens": [_P, _P, _P, c_int, c_int, c_int, _P],
     "mi_begin_step": [_P, _P, _P, c_int, c_int, c_int, _P, _P, _P, c_int, c_int, _P],
     "mi_add_rmsnorm": [c_int, _P, _P, _P, _P, _P, c_int, c_int, c_float, _P, c_int, c_int64, _P],
     "mi_rope_table": [_P, _P, _P, _P, c_int, c_int, _P],
     "mi_rope_kv_write": [
         c_int, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-        c_int, c_int, _P,
+        c_int, c_int, c_int, _P,
     ],
     "mi_silu_mul": [c_int, _P, _P, c_int, c_int, _P],
     "mi_gemm_f32": [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P],
@@ -77,6 +77,21 @@ _SIGNATURES: dict[str, list] = {
     "mi_gemm_skinny_gelu_table_bf16": [_P, c_int64, _P, c_int64, _P, c_int64, _P, c_int, c_int, _P, c_int64, c_int, c_int, c_int, _P],
     "mi_poly_norm": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, _P],
     "mi_gated_table_rows": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
+    "mi_attn_general": [
+        c_int, _P, c_int64, _P, _P, _P, c_int, _P, _P, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, c_int,
+        c_int64, c_int, c_int, c_float, c_int, c_int, _P, c_int, c_float, _P,
+    ],
+    "mi_stream_update_norm": [c_int, _P, c_int64, _P, c_int64, _P, _P, c_float, _P, _P, _P, _P, c_int, c_int, c_float, _P],
+    "mi_clamped_glu": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_float, _P],
+    "mi_short_conv": [c_int, _P, c_int64, _P, _P, c_int64, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P],
+    "mi_gated_delta": [
+        c_int, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int64, _P, _P, _P, c_int64,
+        c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
+    ],
+    "mi_latent_prepare": [
+        c_int, _P, c_int64, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
+        c_float, _P,
+    ],
 }
 
 

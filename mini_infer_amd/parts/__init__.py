@@ -1,6 +1,8 @@
 """Parts a layer is put together from.  Importing this package registers the built-in kinds."""
 
-from mini_infer_amd.parts import attention, block, embedding, feed_forward, norm, position, recurrent  # noqa: F401
+from mini_infer_amd.parts import (  # noqa: F401
+    attention, block, embedding, feed_forward, latent_attention, norm, position, recurrent,
+)
 from mini_infer_amd.parts.base import (
     Block,
     CacheNeeds,

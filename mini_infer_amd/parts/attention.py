@@ -48,7 +48,12 @@ class GQAttention(Mixer):
         scale: float | None = None,
         names: tuple[str, str, str, str] = ("q_proj", "k_proj", "v_proj", "o_proj"),
         suffix: str = ".weight",
+        v_head_dim: int | None = None,
+        sink_logit: float | None = None,
     ) -> None:
+        """`v_head_dim`: value heads of another width than the query and key heads (`head_dim`).
+        `sink_logit`: the softmax's denominator gets one more term exp(sink_logit), a sink that
+        takes weight off the keys and carries no value (0.0: "one added to the denominator")."""
         super().__init__(dtype, device)
         if num_heads % num_kv_heads != 0:
             raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
@@ -63,6 +68,12 @@ class GQAttention(Mixer):
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
         self.head_dim = head_dim
+        self.v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        if self.v_head_dim <= 0 or self.v_head_dim % ops.ATTENTION_HEAD_DIM_STEP != 0:
+            raise ValueError(f"v_head_dim={self.v_head_dim}: the attention kernels take even value head sizes")
+        self.sink_logit = None if sink_logit is None else float(sink_logit)
+        # what the matrix-core kernel and the fused few-row kernels know: no sink, values as wide as keys
+        self._plain_softmax = self.sink_logit is None and self.v_head_dim == head_dim
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
@@ -74,11 +85,12 @@ class GQAttention(Mixer):
             raise ValueError(f"score slopes must be float32 [{num_heads}], got {self.slopes.dtype} {tuple(self.slopes.shape)}")
         q_width, kv_width = num_heads * head_dim, num_kv_heads * head_dim
         self.qkv = self._input_projection(hidden_size, q_width, kv_width, names, suffix)
-        self.out = Linear(q_width, hidden_size, names[3], dtype, device, suffix=suffix)
+        self.out = Linear(num_heads * self.v_head_dim, hidden_size, names[3], dtype, device, suffix=suffix)
 
     def _input_projection(self, hidden_size: int, q_width: int, kv_width: int, names, suffix: str) -> Linear:
         """The stacked product that feeds the attention: q | k | v here."""
-        return Linear(hidden_size, [q_width, kv_width, kv_width], list(names[:3]), self.dtype, self.device, suffix=suffix)
+        v_width = self.num_kv_heads * self.v_head_dim
+        return Linear(hidden_size, [q_width, kv_width, v_width], list(names[:3]), self.dtype, self.device, suffix=suffix)
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
         return {**self.qkv.param_specs(prefix), **self.out.param_specs(prefix)}
@@ -93,6 +105,7 @@ class GQAttention(Mixer):
         layout = self.position.rotary_layout() if self.position is not None else None
         return (
             self.dtype == torch.bfloat16
+            and self._plain_softmax
             and layout == (self.head_dim, False)
             and self.head_dim % 32 == 0
             and ops.scaled_rows_product_takes(rows, self.qkv.weight, self.hidden_size)
@@ -101,9 +114,13 @@ class GQAttention(Mixer):
     def cache_needs(self, page_size: int) -> CacheNeeds:
         # values lie transposed inside a page where the matrix-core kernel will read them
         # (that kernel knows no score bias: such layers keep the plain layout and kernel)
-        transposed = self.slopes is None and ops.mfma_attention_supported(self.dtype, self.head_dim, page_size)
+        transposed = (
+            self.slopes is None and self._plain_softmax
+            and ops.mfma_attention_supported(self.dtype, self.head_dim, page_size)
+        )
+        v_head_dim = None if self.v_head_dim == self.head_dim else self.v_head_dim
         return CacheNeeds(
-            pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_transposed=transposed)
+            pages=PagedKVNeeds(self.num_kv_heads, self.head_dim, self.window, v_head_dim=v_head_dim, v_transposed=transposed)
         )
 
     def forward(
@@ -115,10 +132,11 @@ class GQAttention(Mixer):
         rotary = self.position.rotary(ctx) if self.position is not None else None
         if isinstance(x, ops.ScaledRows) and not (
             rotary is not None
+            and self._plain_softmax
             and ops.qkv_rope_write_takes(x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved)
         ):
             x = x.finish()  # rows but for their norm factors, and no kernel here that applies them
-        if rotary is not None and ops.qkv_rope_write_takes(
+        if rotary is not None and self._plain_softmax and ops.qkv_rope_write_takes(
             x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved
         ):
             # few rows (decode): projection, rotation and cache write are one kernel
@@ -146,6 +164,7 @@ class GQAttention(Mixer):
             qkv, cos, sin, slots, cache.k_pages, cache.v_pages,
             q_heads=self.num_heads, kv_heads=kv_heads, head_dim=self.head_dim,
             rotary_dim=rotary_dim, interleaved=interleaved, v_transposed=cache.v_transposed,
+            v_head_dim=self.v_head_dim,
         )
         return self._project(self._attend(qkv, ctx, cache))
 
@@ -155,7 +174,7 @@ class GQAttention(Mixer):
         assert self.out.weight is not None
         if self.emit_pending_output and self.dtype == torch.bfloat16:
             rows = attended.tokens if isinstance(attended, ops.AttentionPieces) else attended.shape[0]
-            q_width = self.num_heads * self.head_dim
+            q_width = self.num_heads * self.v_head_dim
             if ops.pending_product_pays(rows, self.hidden_size, q_width, self.emit_partial_sums):
                 return ops.PendingProduct(attended, self.out.weight)
         if isinstance(attended, ops.AttentionPieces):
@@ -166,12 +185,16 @@ class GQAttention(Mixer):
         """Attention of the rotated queries (the first columns of `queries`) over the cache pages.
         At the smallest batches the key ranges may come back uncombined, for the output
         projection to combine on its way (one launch less a layer)."""
-        few = queries.dtype == torch.bfloat16 and ops.attention_pieces_pay(ctx.num_tokens, self.num_heads, self.head_dim)
+        few = (
+            queries.dtype == torch.bfloat16 and self._plain_softmax
+            and ops.attention_pieces_pay(ctx.num_tokens, self.num_heads, self.head_dim)
+        )
         return ops.paged_attention(
             queries, cache.k_pages, cache.v_pages, ctx.block_tables[cache.group], ctx.token_request,
             ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=self.num_heads,
             kv_heads=self.num_kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
             max_seq_len=ctx.max_seq_len, v_transposed=cache.v_transposed, combine=not few, slopes=self.slopes,
+            v_head_dim=self.v_head_dim, sink_logit=self.sink_logit,
         )
 
 
@@ -260,6 +283,9 @@ def build_gqa_attention(desc: dict, dtype: torch.dtype, device, shared: dict | N
             position = POSITION_ENCODINGS.lookup(pos_desc["kind"])(pos_desc, dtype, device, shared)
             if shared is not None:
                 shared[key] = position
+    extra = {k: desc[k] for k in ("suffix", "v_head_dim", "sink_logit") if k in desc}
+    if "names" in desc:
+        extra["names"] = tuple(desc["names"])
     return GQAttention(
         int(desc["hidden_size"]),
         int(desc["num_heads"]),
@@ -270,4 +296,5 @@ def build_gqa_attention(desc: dict, dtype: torch.dtype, device, shared: dict | N
         device,
         window=desc.get("window"),
         scale=desc.get("scale"),
+        **extra,
     )

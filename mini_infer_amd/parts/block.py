@@ -123,6 +123,76 @@ def build_pre_norm_block(desc: dict, dtype: torch.dtype, device, shared: dict | 
     )
 
 
+class ParallelBlock(Block):
+    """One norm, and every sublayer reads its output; their results are added to the stream
+    together, scaled by one number:
+
+        h = norm(x);    x <- x + scale * (mixer(h) + feed_forward(h))       (a layer may have no feed-forward)
+
+    The add is left to whatever norm comes next, as `ops.StreamUpdate` (with the bias of the
+    feed-forward's last product, where it has one, riding along): a norm that knows such an
+    update makes it in the launch that also begins the next layer."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, feed_forward: FeedForward | None, scale: float,
+                 names: dict[str, str], dtype: torch.dtype, device) -> None:
+        super().__init__(dtype, device)
+        self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+        self.scale, self.names = float(scale), names
+
+    def _children(self):
+        parts = [(self.names["norm"], self.norm), (self.names["mixer"], self.mixer)]
+        if self.feed_forward is not None:
+            parts.append((self.names["feed_forward"], self.feed_forward))
+        return parts
+
+    @property
+    def graph_safe(self) -> bool:  # type: ignore[override]
+        return all(part.graph_safe for _, part in self._children())
+
+    @property
+    def takes_pending_products(self) -> bool:  # type: ignore[override]
+        return self.norm.takes_pending_products
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        specs: dict[str, ParamSpec] = {}
+        for sub, part in self._children():
+            specs.update(part.param_specs(prefix + sub))
+        return specs
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        for sub, part in self._children():
+            part.load_params(prefix + sub, get)
+
+    def forward(self, delta, residual: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        from mini_infer_amd import ops
+
+        h = self.norm.forward(delta, residual)
+        if hasattr(h, "finish"):
+            h = h.finish()
+        mixed = self.mixer.forward(h, ctx, cache, writes_cache)
+        mixed = mixed.finish() if hasattr(mixed, "finish") else mixed
+        fed = bias = None
+        if self.feed_forward is not None:
+            fed = self.feed_forward.forward(h, ctx)
+            fed = fed.finish() if hasattr(fed, "finish") else fed
+            bias = getattr(self.feed_forward, "output_bias", None)
+        return ops.StreamUpdate(mixed, fed, bias, None, self.scale)
+
+
+@register_block("parallel")
+def build_parallel_block(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ParallelBlock:
+    """`desc`: `norm`, `mixer`, optional `feed_forward` (descriptions with a `kind`), `scale` (the
+    number the sublayers' sum is multiplied with before it is added) and `names`."""
+    shared = {} if shared is None else shared
+    ffn = desc.get("feed_forward")
+    return ParallelBlock(
+        NORMS.lookup(desc["norm"]["kind"])(desc["norm"], dtype, device, shared),
+        MIXERS.lookup(desc["mixer"]["kind"])(desc["mixer"], dtype, device, shared),
+        FEED_FORWARDS.lookup(ffn["kind"])(ffn, dtype, device, shared) if ffn is not None else None,
+        float(desc.get("scale", 1.0)), dict(desc["names"]), dtype, device,
+    )
+
+
 class OutputNormBlock(Block):
     """Sublayers that read the stream itself and are normed on the way OUT:
 

@@ -40,6 +40,18 @@ class TokenEmbedding(Embedding):
         return ops.embed_gather(self.weight, ctx.token_ids)
 
 
+class ScaledEmbedding(TokenEmbedding):
+    """`table[token] * scale`."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, name: str, scale: float, dtype: torch.dtype, device) -> None:
+        super().__init__(vocab_size, hidden_size, name, dtype, device)
+        self.scale = float(scale)
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        assert self.weight is not None, "embedding used before its table was loaded"
+        return ops.embed_gather(self.weight, ctx.token_ids, self.scale)
+
+
 SINUSOID_BASE = 10000.0
 STREAM_CAST = "stream_cast"  # key in `StepContext.shared`: (the stream, its latest copy in the compute dtype)
 
@@ -130,6 +142,11 @@ class OutputHead(Head):
 @register_embedding("token_embedding")
 def build_token_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> TokenEmbedding:
     return TokenEmbedding(int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), dtype, device)
+
+
+@register_embedding("scaled_embedding")
+def build_scaled_embedding(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ScaledEmbedding:
+    return ScaledEmbedding(int(desc["vocab_size"]), int(desc["hidden_size"]), str(desc["name"]), float(desc["scale"]), dtype, device)
 
 
 @register_embedding("scaled_sinusoid_embedding")

@@ -177,3 +177,66 @@ def build_token_side_input(desc: dict, dtype: torch.dtype, device, shared: dict 
     if "names" in extra:
         extra["names"] = tuple(extra["names"])
     return TokenSideInput(int(desc["hidden_size"]), int(desc["dim"]), int(desc["first_col"]), table, dtype, device, **extra)
+
+
+GATE_SLOPE = 1.702  # of the logistic that gates: g * logistic(1.702 g) approximates gelu(g)
+
+
+class ClampedGatedFeedForward(FeedForward):
+    """Gated, with biases on all three products and both branches clamped before they meet:
+
+        g = min(W_gate x + b_gate, limit)          u = clamp(W_up x + b_up, -limit, limit)
+        y = W_down (g * logistic(slope * g) * (u + 1)) + b_down
+
+    Gate and up are stacked at load so one product yields [gate | up]; their biases and the
+    activation are one kernel.  The down product's bias is not added here: `forward` returns the
+    product, and `output_bias` (float32) is for whoever adds the result to the stream to add with
+    it (`ops.StreamUpdate.bias`)."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, dtype: torch.dtype, device, *,
+                 slope: float = GATE_SLOPE, names: tuple[str, str, str] = ("gate", "up", "down"), suffix: str = "",
+                 bias_suffix: str = ".b") -> None:
+        super().__init__(dtype, device)
+        if limit <= 0:
+            raise ValueError(f"clamped gated feed-forward: the limit must be positive, got {limit}")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.limit, self.slope = float(limit), float(slope)
+        self.names, self.suffix, self.bias_suffix = tuple(names), suffix, bias_suffix
+        self.gate_up = Linear(hidden_size, [intermediate_size, intermediate_size], [names[0], names[1]], dtype, device, suffix=suffix)
+        self.down = Linear(intermediate_size, hidden_size, names[2], dtype, device, suffix=suffix)
+        self.gate_up_bias: torch.Tensor | None = None
+        self.output_bias: torch.Tensor | None = None
+
+    def _bias_name(self, prefix: str, which: int) -> str:
+        return prefix + self.names[which] + self.suffix + self.bias_suffix
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {
+            **self.gate_up.param_specs(prefix), **self.down.param_specs(prefix),
+            self._bias_name(prefix, 0): ParamSpec((self.intermediate_size,), dtype="float32"),
+            self._bias_name(prefix, 1): ParamSpec((self.intermediate_size,), dtype="float32"),
+            self._bias_name(prefix, 2): ParamSpec((self.hidden_size,), dtype="float32"),
+        }
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.gate_up.load_params(prefix, get)
+        self.down.load_params(prefix, get)
+        self.gate_up_bias = torch.cat([get(self._bias_name(prefix, 0)).float(), get(self._bias_name(prefix, 1)).float()]).contiguous()
+        self.output_bias = get(self._bias_name(prefix, 2)).float().contiguous()
+
+    def forward(self, x, ctx: StepContext) -> torch.Tensor:
+        assert self.gate_up_bias is not None, "feed-forward used before its weights were loaded"
+        if isinstance(x, ops.ScaledRows):
+            x = x.finish()
+        act = ops.clamped_glu(self.gate_up.forward(x), self.gate_up_bias, self.limit, self.slope)
+        return self.down.forward(act)
+
+
+@register_feed_forward("clamped_glu")
+def build_clamped_gated_feed_forward(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> ClampedGatedFeedForward:
+    extra = {k: desc[k] for k in ("slope", "suffix", "bias_suffix") if k in desc}
+    if "names" in desc:
+        extra["names"] = tuple(desc["names"])
+    return ClampedGatedFeedForward(int(desc["hidden_size"]), int(desc["intermediate_size"]), float(desc["limit"]), dtype, device, **extra)

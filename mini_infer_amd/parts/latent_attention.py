@@ -1,0 +1,142 @@
+"""Attention over one small latent row per token.
+
+Every head's keys and values are linear maps of a latent `c` of `kv_rank` numbers per token;
+beside it one rotated key part `r` of `rot_dim` numbers is shared by all heads:
+
+    [x_c | x_r] = W_dkv h        c = rms_norm(x_c) * w_c        r = rotate(x_r, position)
+    q_a = W_q h  laid out per head as [plain (head_dim) | to rotate (rot_dim)]
+    score_a(i, j) = (q_a,plain(i) . W_uk,a c(j) + rotate(q_a,rot(i)) . r(j)) * scale
+    out = W_o concat_a( sum_j softmax_j(score_a(i, .)) W_uv,a c(j) )
+
+Only `[c | r]` is cached: one key head of `kv_rank + rot_dim` numbers a token, whatever the
+number of heads.  The key map is folded into the query, `q'_a = W_uk,a^T q_a,plain`, so a
+head's score is `[q'_a | q_a,rot] . [c | r]`, and the value map is applied after the
+attention, `W_uv,a (sum_j p_j c(j))`: the attention itself is the paged kernel with a single
+key/value head whose value row is the front part of its key row.  Prompts and single tokens
+take the same path, so a position's result does not depend on how its prompt was cut.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from mini_infer_amd import ops
+from mini_infer_amd.parts.base import (
+    CacheNeeds,
+    LayerCache,
+    Mixer,
+    PagedKVNeeds,
+    ParamSpec,
+    PositionEncoding,
+    StepContext,
+    TensorGetter,
+)
+from mini_infer_amd.parts.linear import Linear
+from mini_infer_amd.registry import POSITION_ENCODINGS, register_mixer
+
+DEFAULT_NAMES = {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_k": "uk", "up_v": "uv", "out": "o"}
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, v_head_dim: int, kv_rank: int,
+                 position: PositionEncoding, scale: float, norm_eps: float, dtype: torch.dtype, device, *,
+                 names: dict[str, str] | None = None, suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        for what, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim),
+                            ("v_head_dim", v_head_dim), ("kv_rank", kv_rank)):
+            if value <= 0:
+                raise ValueError(f"latent attention: {what} must be positive, got {value}")
+        if rot_dim < 0 or rot_dim % 2 or kv_rank % 2:
+            raise ValueError(f"latent attention: rot_dim={rot_dim} and kv_rank={kv_rank} must be even")
+        layout = position.rotary_layout()
+        if layout != (rot_dim, True):
+            raise ValueError(f"latent attention rotates {rot_dim} entries in neighbouring pairs; the encoding gives {layout}")
+        if kv_rank + rot_dim > ops.kernels.GENERAL_ATTENTION_MAX_KEY_DIM or kv_rank > ops.kernels.GENERAL_ATTENTION_MAX_VALUE_DIM:
+            raise ValueError(
+                f"latent attention: cached rows of {kv_rank} + {rot_dim} exceed what the attention kernel takes "
+                f"({ops.kernels.GENERAL_ATTENTION_MAX_VALUE_DIM} for the latent, {ops.kernels.GENERAL_ATTENTION_MAX_KEY_DIM} in all)"
+            )
+        self.hidden_size, self.num_heads, self.head_dim, self.rot_dim = hidden_size, num_heads, head_dim, rot_dim
+        self.v_head_dim, self.kv_rank = v_head_dim, kv_rank
+        self.position, self.scale, self.norm_eps = position, float(scale), float(norm_eps)
+        self.names = {**DEFAULT_NAMES, **(names or {})}
+        n = self.names
+        self.q_head_width = head_dim + rot_dim
+        # one product yields [q of every head | x_c | x_r]
+        self.q_down = Linear(hidden_size, [num_heads * self.q_head_width, kv_rank + rot_dim], [n["q"], n["down"]], dtype,
+                             device, suffix=suffix)
+        self.up_k = Linear(kv_rank, num_heads * head_dim, n["up_k"], dtype, device, suffix=suffix)
+        self.up_v = Linear(kv_rank, num_heads * v_head_dim, n["up_v"], dtype, device, suffix=suffix)
+        self.out = Linear(num_heads * v_head_dim, hidden_size, n["out"], dtype, device, suffix=suffix)
+        self.latent_norm: torch.Tensor | None = None
+        self.fold_k: torch.Tensor | None = None  # [heads, kv_rank, head_dim]: W_uk,a transposed
+        self.map_v: torch.Tensor | None = None  # [heads, v_head_dim, kv_rank]
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        return {
+            **self.q_down.param_specs(prefix), **self.up_k.param_specs(prefix), **self.up_v.param_specs(prefix),
+            **self.out.param_specs(prefix),
+            prefix + self.names["down_norm"]: ParamSpec((self.kv_rank,), init="norm_weight", dtype="float32"),
+        }
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        self.q_down.load_params(prefix, get)
+        self.up_k.load_params(prefix, get)
+        self.up_v.load_params(prefix, get)
+        self.out.load_params(prefix, get)
+        self.latent_norm = get(prefix + self.names["down_norm"]).float().contiguous()
+        assert self.up_k.weight is not None and self.up_v.weight is not None
+        self.fold_k = self.up_k.weight.view(self.num_heads, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.map_v = self.up_v.weight.view(self.num_heads, self.v_head_dim, self.kv_rank)
+        self.up_k.weight = None  # (kept transposed only)
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        # one key head, rows [c | r]; the values are the rows' front part: no value pages
+        return CacheNeeds(pages=PagedKVNeeds(1, self.kv_rank + self.rot_dim, None, v_head_dim=0))
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
+        assert cache.group is not None and cache.k_pages is not None
+        assert self.fold_k is not None and self.map_v is not None and self.latent_norm is not None, \
+            "latent attention used before its weights were loaded"
+        if hasattr(x, "finish"):
+            x = x.finish()
+        heads, rank, rot, width = self.num_heads, self.kv_rank, self.rot_dim, self.kv_rank + self.rot_dim
+        proj = self.q_down.forward(x)
+        tokens = proj.shape[0]
+        rotary = self.position.rotary(ctx)
+        queries = torch.empty((tokens, heads * width), dtype=proj.dtype, device=proj.device)
+        ops.latent_prepare(
+            proj, rotary.cos, rotary.sin, self.latent_norm, ctx.slot_mapping[cache.group] if writes_cache else None,
+            cache.k_pages, queries, heads=heads, q_head_width=self.q_head_width, q_rot_at=self.head_dim,
+            c_col=heads * self.q_head_width, rank=rank, rot=rot, eps=self.norm_eps,
+        )
+        # the key map folded into the queries: q'_a = W_uk,a^T q_a,plain
+        plain = proj[:, : heads * self.q_head_width].unflatten(1, (heads, self.q_head_width))[:, :, : self.head_dim]
+        ops.linear_per_head(plain, self.fold_k, queries.unflatten(1, (heads, width))[:, :, :rank])
+        mixed = ops.paged_attention(
+            queries, cache.k_pages, None, ctx.block_tables[cache.group], ctx.token_request, ctx.positions,
+            ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=heads, kv_heads=1, head_dim=width, scale=self.scale,
+            window=None, max_seq_len=ctx.max_seq_len, v_head_dim=rank,
+        )
+        # the value map after the attention: W_uv,a (sum_j p_j c_j)
+        values = torch.empty((tokens, heads * self.v_head_dim), dtype=proj.dtype, device=proj.device)
+        ops.linear_per_head(mixed.unflatten(1, (heads, rank)), self.map_v, values.unflatten(1, (heads, self.v_head_dim)))
+        return self.out.forward(values)
+
+
+@register_mixer("latent_attention")
+def build_latent_attention(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> LatentAttention:
+    pos_desc = desc["position"]
+    key = ("position", repr(sorted(pos_desc.items(), key=lambda kv: kv[0])))
+    position = shared.get(key) if shared is not None else None
+    if position is None:
+        position = POSITION_ENCODINGS.lookup(pos_desc["kind"])(pos_desc, dtype, device, shared)
+        if shared is not None:
+            shared[key] = position
+    return LatentAttention(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["head_dim"]), int(desc["rot_dim"]),
+        int(desc["v_head_dim"]), int(desc["kv_rank"]), position, float(desc["scale"]), float(desc["norm_eps"]), dtype, device,
+        names=desc.get("names"), suffix=str(desc.get("suffix", "")),
+    )

@@ -50,6 +50,10 @@ class RMSNorm(Norm):
         rows: torch.Tensor | None = None,
     ) -> "torch.Tensor | ops.ScaledRows":
         assert self.weight is not None, "RMSNorm used before its weight was loaded"
+        if isinstance(delta, ops.StreamUpdate):
+            # the sublayers' outputs of a layer that adds them together, scaled: the add and
+            # the norm are one launch
+            return ops.stream_update_norm(delta, residual, self.weight, self.eps, rows)
         if isinstance(delta, ops.PendingProduct):
             # few rows: the product, the add and the norm but for the rows' factors are one
             # kernel, if the part that follows has a kernel that applies the factors in this step

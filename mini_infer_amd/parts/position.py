@@ -25,6 +25,13 @@ def default_inv_freq(rotary_dim: int, theta: float) -> torch.Tensor:
     return 1.0 / (theta**exponent)
 
 
+def exact_inv_freq(rotary_dim: int, theta: float) -> torch.Tensor:
+    """theta^(-2j/D) evaluated in 64-bit and rounded to float32 once (`default_inv_freq` makes
+    the same table in float32 arithmetic, as the reference does, and is a last bit or two off)."""
+    exponent = torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim
+    return torch.pow(torch.tensor(float(theta), dtype=torch.float64), -exponent).to(torch.float32)
+
+
 def llama3_inv_freq(
     inv_freq: torch.Tensor,
     factor: float,
@@ -61,6 +68,7 @@ class RotaryPosition(PositionEncoding):
         rotary_dim: int | None = None,
         interleaved: bool = False,
         llama3: dict | None = None,
+        exact_frequencies: bool = False,
     ) -> None:
         super().__init__(dtype, device)
         self.head_dim = head_dim
@@ -68,7 +76,7 @@ class RotaryPosition(PositionEncoding):
         if self.rotary_dim % 2 != 0 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim={self.rotary_dim} must be even and within head_dim={head_dim}")
         self.interleaved = bool(interleaved)
-        table = default_inv_freq(self.rotary_dim, float(theta))
+        table = (exact_inv_freq if exact_frequencies else default_inv_freq)(self.rotary_dim, float(theta))
         if llama3 is not None:
             table = llama3_inv_freq(
                 table,
@@ -111,4 +119,5 @@ def build_rotary(desc: dict, dtype: torch.dtype, device, shared: dict | None = N
         rotary_dim=desc.get("rotary_dim"),
         interleaved=bool(desc.get("interleaved", False)),
         llama3=desc.get("llama3"),
+        exact_frequencies=bool(desc.get("exact_frequencies", False)),
     )

@@ -1,6 +1,6 @@
 """Recurrent mixers: state of fixed size per request instead of pages of keys and values.
 
-`MinGRU` is a gated recurrence whose gates read only the current token, so all gates of a
+`GatedDeltaRule` (below) keeps a matrix per head that is written by the delta rule.  `MinGRU` is a gated recurrence whose gates read only the current token, so all gates of a
 portion come from one stacked product and only the recurrence itself walks the tokens:
 
     z_t = sigmoid(W_z h_t + b_z)        u_t = W_x h_t + b_x
@@ -93,3 +93,112 @@ class MinGRU(Mixer):
 def build_min_gru(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> MinGRU:
     return MinGRU(int(desc["hidden_size"]), int(desc["width"]), dtype, device, names=desc.get("names"),
                   suffix=str(desc.get("suffix", "")))
+
+
+DELTA_NAMES = {
+    "q": "q", "k": "k", "v": "v", "write": "b", "decay": "a", "gate": "g", "out": "o", "conv": ".conv",
+    "rate": "A_log", "step_bias": "dt_bias", "norm": "norm",
+}
+DELTA_UNIT_NORM_EPS = 1e-6  # inside the root that makes q and k unit vectors (fixed by the kernel)
+
+
+class GatedDeltaRule(Mixer):
+    """A matrix state S (head_dim x v_head_dim, float32) per head, written by the gated delta rule:
+
+        q, k, v = silu(short_conv(W_q h)), silu(short_conv(W_k h)), silu(short_conv(W_v h))
+        q, k  <- unit vectors per head (q also times head_dim^-1/2)
+        w_t = logistic(W_b h)                  d_t = exp(-exp(A) * softplus(W_a h + bias))   (per head)
+        S <- d_t S;   u = w_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
+        y_t = W_o (rms_norm(o_t) * weight * silu(W_g h))
+
+    with `num_kv_heads` heads of q and k shared by groups of the `num_heads` value heads.  A
+    request's S and the last taps-1 inputs of the three convolutions live in its state slot."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int, taps: int,
+                 norm_eps: float, dtype: torch.dtype, device, *, names: dict[str, str] | None = None, suffix: str = "") -> None:
+        super().__init__(dtype, device)
+        for what, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads),
+                            ("head_dim", head_dim), ("v_head_dim", v_head_dim), ("taps", taps)):
+            if value <= 0:
+                raise ValueError(f"gated delta rule: {what} must be positive, got {value}")
+        if num_heads % num_kv_heads != 0:
+            raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
+        if head_dim > 256 or v_head_dim > 256 or taps > 16:
+            raise ValueError(f"gated delta rule: the kernels take heads up to 256 x 256 and 16 taps, got {head_dim} x {v_head_dim}, {taps}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.v_head_dim, self.taps, self.norm_eps = head_dim, v_head_dim, taps, float(norm_eps)
+        self.names = {**DELTA_NAMES, **(names or {})}
+        self.suffix = suffix
+        n = self.names
+        qk, vw = num_kv_heads * head_dim, num_heads * v_head_dim
+        self.channels = 2 * qk + vw  # what passes the convolution: q | k | v
+        # one product yields [q | k | v | write | decay | gate] for every token of the step
+        self.inputs = Linear(hidden_size, [qk, qk, vw, num_heads, num_heads, vw],
+                             [n["q"], n["k"], n["v"], n["write"], n["decay"], n["gate"]], dtype, device, suffix=suffix)
+        self.col_write, self.col_decay, self.col_gate = self.channels, self.channels + num_heads, self.channels + 2 * num_heads
+        self.out = Linear(vw, hidden_size, n["out"], dtype, device, suffix=suffix)
+        self.conv_weight: torch.Tensor | None = None  # float32 [channels, taps]
+        self.rate: torch.Tensor | None = None
+        self.step_bias: torch.Tensor | None = None
+        self.norm_weight: torch.Tensor | None = None
+
+    def _conv_names(self, prefix: str) -> list[tuple[str, int]]:
+        n, qk = self.names, self.num_kv_heads * self.head_dim
+        return [(prefix + n[part] + self.suffix + n["conv"], rows)
+                for part, rows in (("q", qk), ("k", qk), ("v", self.num_heads * self.v_head_dim))]
+
+    def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
+        n = self.names
+        specs = {**self.inputs.param_specs(prefix), **self.out.param_specs(prefix)}
+        for name, rows in self._conv_names(prefix):
+            specs[name] = ParamSpec((rows, self.taps), dtype="float32")
+        specs[prefix + n["rate"]] = ParamSpec((self.num_heads,), dtype="float32")
+        specs[prefix + n["step_bias"]] = ParamSpec((self.num_heads,), dtype="float32")
+        specs[prefix + n["norm"]] = ParamSpec((self.v_head_dim,), init="norm_weight", dtype="float32")
+        return specs
+
+    def load_params(self, prefix: str, get: TensorGetter) -> None:
+        n = self.names
+        self.inputs.load_params(prefix, get)
+        self.out.load_params(prefix, get)
+        self.conv_weight = torch.cat([get(name).float() for name, _ in self._conv_names(prefix)], dim=0).contiguous()
+        self.rate = get(prefix + n["rate"]).float().contiguous()
+        self.step_bias = get(prefix + n["step_bias"]).float().contiguous()
+        self.norm_weight = get(prefix + n["norm"]).float().contiguous()
+
+    def cache_needs(self, page_size: int) -> CacheNeeds:
+        state = {"recurrent": StateNeeds(ops.delta_state_shape(self.num_heads, self.head_dim, self.v_head_dim), torch.float32)}
+        if self.taps > 1:
+            state["tail"] = StateNeeds((self.taps - 1, self.channels), self.dtype)
+        return CacheNeeds(state=state)
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True) -> torch.Tensor:
+        if not writes_cache:
+            raise NotImplementedError("a recurrent mixer owns its state; it cannot read another call's")
+        assert self.conv_weight is not None and self.rate is not None, "gated delta rule used before its weights were loaded"
+        assert isinstance(cache.state, dict), "the gated delta rule needs its state rows from the cache manager"
+        if hasattr(x, "finish"):
+            x = x.finish()
+        proj = self.inputs.forward(x)
+        if self.taps > 1:
+            tail = cache.state["tail"]
+        else:  # (no taps before the current one: nothing to remember)
+            tail = torch.empty((2, 0, self.channels), dtype=proj.dtype, device=proj.device)
+        qkv = ops.short_conv(proj, self.channels, self.conv_weight, tail, ctx.cu_seqlens_q, ctx.state_slots, ctx.token_request)
+        mixed = ops.gated_delta(
+            qkv, proj, self.col_write, self.col_decay, self.col_gate, self.rate, self.step_bias, self.norm_weight,
+            cache.state["recurrent"], ctx.cu_seqlens_q, ctx.state_slots, heads=self.num_heads, kv_heads=self.num_kv_heads,
+            dim=self.head_dim, vdim=self.v_head_dim, eps=self.norm_eps,
+        )
+        return self.out.forward(mixed)
+
+
+@register_mixer("gated_delta_rule")
+def build_gated_delta_rule(desc: dict, dtype: torch.dtype, device, shared: dict | None = None) -> GatedDeltaRule:
+    return GatedDeltaRule(
+        int(desc["hidden_size"]), int(desc["num_heads"]), int(desc["num_kv_heads"]), int(desc["head_dim"]),
+        int(desc["v_head_dim"]), int(desc["taps"]), float(desc["norm_eps"]), dtype, device, names=desc.get("names"),
+        suffix=str(desc.get("suffix", "")),
+    )
