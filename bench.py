@@ -434,6 +434,25 @@ def nadosun_config(sizes: dict, layers: int) -> dict:
             "layers": [attention if i % 3 == 2 else recurrent for i in range(layers)]}
 
 
+def zekonex_config(sizes: dict, layers: int) -> dict:
+    """A Zekonex model with the widths of a Llama configuration: gated delta rule layers alternating
+    with latent attention layers, every fourth layer grouped-query attention with a sink; every layer
+    with a clamped gated feed-forward of Llama's width beside its mixer.  The delta layers have Llama's
+    query heads as value heads and its key/value heads as query/key heads; the latent is four head
+    sizes wide with half a head size of rotated part (the proportions of published latent-attention models)."""
+    h, heads, kv, d = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"], sizes["head_dim"]
+    mlp = {"kind": "dense", "ff": sizes["intermediate_size"], "limit": 7.0}
+    attention = {"type": "attention", "mlp": mlp,
+                 "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "rot": {"base": 500000.0, "dims": d // 2}}}
+    delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4}}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": d, "rot_dim": d // 2, "vdim": d, "kv_rank": 4 * d, "scale": (d + d // 2) ** -0.5,
+                        "rot": {"base": 10000.0, "dims": d // 2}}}
+    return {"architecture": "Zekonex", "vocab": sizes["vocab_size"], "width": h, "embedding": {"scale": float(h) ** 0.5},
+            "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "layers": [(delta, latent, delta, attention)[i % 4] for i in range(layers)]}
+
+
 def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
     """What a step must move and compute, from the model's own list of tensors: bytes of every matrix
     a decode step streams (tables that are only gathered from are left out), multiply-adds of its
@@ -444,6 +463,23 @@ def model_costs(model, raw: dict, tokens: int, context: float) -> dict:
     if "lm_head.weight" not in specs and "head" not in specs:  # a tied head streams the embedding's table
         matrix += int(specs["model.embed_tokens.weight"].shape[0]) * int(specs["model.embed_tokens.weight"].shape[1])
     head = int(model.vocab_size) * int(model.spec.hidden_size)
+    state_bytes = 0
+    if raw.get("architecture") == "Zekonex":
+        # attention: keys and values of every key/value head; latent attention: one row [latent | rotated
+        # part] per token for all heads, scored against and summed over by every head in the latent's width;
+        # delta rule: no keys, a float32 matrix per head read and written once a step
+        mixers = [(l["type"], l["mixer"]) for l in raw["layers"]]
+        kv_values = sum(m["kv_heads"] * (m["dim"] + m["vdim"]) * context for t, m in mixers if t == "attention")
+        kv_values += sum((m["kv_rank"] + m["rot_dim"]) * context for t, m in mixers if t == "latent_attention")
+        state_bytes = sum(2 * 4 * m["heads"] * m["dim"] * m["vdim"] for t, m in mixers if t == "delta")
+        pairs_all = tokens * (tokens + 1) / 2
+        attention_flops = sum(2.0 * pairs_all * m["heads"] * (m["dim"] + m["vdim"]) for t, m in mixers if t == "attention")
+        attention_flops += sum(2.0 * pairs_all * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"]) for t, m in mixers if t == "latent_attention")
+        # the recurrence: per token and head three passes over dim x vdim (decay and read, write, read out)
+        attention_flops += sum(6.0 * tokens * m["heads"] * m["dim"] * m["vdim"] for t, m in mixers if t == "delta")
+        # (the latent's key and value maps are applied per head to queries and outputs: counted with the matrices)
+        return {"matrix_values": matrix, "kv_values_per_request": kv_values, "state_bytes_per_request": state_bytes,
+                "prefill_flops": 2.0 * tokens * (matrix - head) + 2.0 * head + attention_flops}
     if "layers" in raw:  # Nadosun: windowed layers
         layers = [(m["heads"], m["kv_heads"], m["dim"], m["mask"]["size"]) for m in (l["mixer"] for l in raw["layers"] if l["type"] == "attention")]
     else:
@@ -505,7 +541,7 @@ def measure_model(raw: dict, dtype: str, batches: list[int], steps: int, warmup:
         seconds = (time.perf_counter() - started) / steps
         for rid in ids:
             runner.free_request(rid)
-        moved = (costs["matrix_values"] + batch * costs["kv_values_per_request"]) * elem
+        moved = (costs["matrix_values"] + batch * costs["kv_values_per_request"]) * elem + batch * costs.get("state_bytes_per_request", 0)
         out["decode"][f"b{batch}"] = {"ms_per_step": round(seconds * 1e3, 4), "tok_s": round(batch / seconds, 1),
                                       "frac_of_hbm_peak": round(moved / seconds / 1e9 / PEAK_HBM_GBS, 4)}
     del runner
@@ -517,13 +553,16 @@ def measure_design(design: str, sizes_name: str, dtype: str, layers: int | None,
                    alone: bool = False) -> dict:
     model_name, sizes = SIZES[sizes_name]
     layers = layers if layers is not None else DESIGN_LAYERS
-    if design != "nadosun":
-        raise ValueError(f"no design {design!r} to compare")
-    ours = nadosun_config(sizes, layers)
     theirs = dict(sizes, num_hidden_layers=layers)
+    if design == "nadosun":
+        sides = [(design, nadosun_config(sizes, layers)), ("llama", theirs)]
+    elif design == "zekonex":  # beside the other design of mixed recurrent and attention layers, and beside Llama
+        sides = [(design, zekonex_config(sizes, layers)), ("nadosun", nadosun_config(sizes, layers)), ("llama", theirs)]
+    else:
+        raise ValueError(f"no design {design!r} to compare")
     line = {"design": design, "sizes": f"{model_name} layer sizes", "layers": layers, "dtype": dtype, "window": DESIGN_WINDOW,
             "data": "synthetic: random token ids, random-init weights", "steps": steps, "warmup": warmup}
-    for name, raw in ((design, ours), ("llama", theirs))[: 1 if alone else 2]:
+    for name, raw in sides[: 1 if alone else len(sides)]:
         print(f"bench.py: {name} at {model_name} layer sizes, {layers} layers", file=sys.stderr, flush=True)
         line[name] = measure_model(raw, dtype, batches, steps, warmup)
     return line
@@ -566,10 +605,10 @@ def main() -> int:
                         help="with --serving / --reference-workload: launch steps that have portions of prompts in them kernel "
                         "by kernel, however few their tokens (recorded steps of single tokens stay)")
     parser.add_argument(
-        "--design", default=None, choices=("nadosun",),
+        "--design", default=None, choices=("nadosun", "zekonex"),
         help="instead of the default run: prefill (one 2,048-token prompt) and decode (batch 1, --batch and 64; --steps "
         "steps, default 64 here) of that design beside Llama at the layer sizes of --sizes and equal depth "
-        "(--layers, default 12); prints one JSON line and exits",
+        "(--layers, default 12; zekonex also beside nadosun); prints one JSON line and exits",
     )
     parser.add_argument("--design-alone", action="store_true", help="with --design: leave the Llama side out (for profiles)")
     parser.add_argument("--attention-batch", type=int, default=0)

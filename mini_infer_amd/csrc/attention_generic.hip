@@ -444,13 +444,14 @@ extern "C" int mi_attn_general(int dtype, const void* q, int64_t q_row_stride, c
 // The combining step alone, for partials written by the matrix-core kernel.
 extern "C" int mi_attn_reduce_bf16(const float* part_acc, const float* part_ml, void* out,
                                    int64_t out_row_stride, int num_tokens, int q_heads,
-                                   int head_dim, int num_splits, hipStream_t stream) {
+                                   int head_dim, int num_splits, int has_sink, float sink_logit,
+                                   hipStream_t stream) {
   if (num_tokens == 0) return MI_OK;
   MI_REQUIRE(q_heads <= 65535, "attn_reduce: too many heads");
   dim3 rgrid(num_tokens, q_heads);
   attn_reduce_kernel<bf16_t><<<rgrid, MI_WAVE, 0, stream>>>(part_acc, part_ml, (bf16_t*)out,
                                                             out_row_stride, q_heads, head_dim,
-                                                            num_splits, 0, 0.f);
+                                                            num_splits, has_sink, sink_logit);
   MI_CHECK_LAUNCH("attn_reduce");
   return MI_OK;
 }

@@ -13,10 +13,11 @@
 //                     and the read-out o divided by its root mean square over vdim, times a weight
 //                     per column and silu(g).
 //
-// The state of a head lies in memory as [ceil(dim/4)][vdim][4]: element (i, j) at
-// ((i / 4) * vdim + j) * 4 + i % 4.  Column j of S is kept by four neighbouring lanes, lane r of
-// them holding rows r, r + 4, ...: a token costs each lane dim/4 multiply-adds per pass and the
-// four partial sums meet through two lane exchanges, with no barrier inside a tile of tokens.
+// The state of a head lies in memory transposed and padded, [vdim][dim_pad].  Column j of S is
+// kept by R neighbouring lanes (4, 8 or 16), each holding a run of its rows: a token costs a lane
+// dim/R multiply-adds per pass and the partial sums meet through register moves between the
+// lanes, with no barrier inside a tile of tokens.  Columns are independent of one another, so a
+// head's work spreads over R * vdim threads however short the step.
 // Everything that enters the recurrence is float32 (the projections and the convolution's
 // outputs are read in the element type); in the 32-bit engine the scalar gates, the unit norms
 // and the read-out's norm are evaluated in 64-bit and rounded once.
@@ -90,9 +91,27 @@ struct TokenGates {
   float decay, write;
 };
 
-// ROWS: rows of S a lane keeps (>= ceil(ceil(dim / 4))).  Block: 4 * vdim threads rounded up to
-// whole waves; thread = 4 * column + r.
-template <typename T, int ROWS>
+// Sum over the R neighbouring lanes that keep one column (R = 4, 8 or 16, inside a row of 16
+// lanes); every lane gets the total.  Lane exchanges inside a row are register moves (DPP):
+// neighbours, pairs, then the mirror image inside 8 and inside 16 lanes, which after the first
+// two steps holds the other half's sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int R>
+__device__ __forceinline__ float lanes_sum(float v) {
+  v += dpp_move<0xB1>(v);  // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);  // quad_perm [2,3,0,1]
+  if constexpr (R >= 8) v += dpp_move<0x141>(v);   // row_half_mirror
+  if constexpr (R >= 16) v += dpp_move<0x140>(v);  // row_mirror
+  return v;
+}
+
+// R lanes keep a column of S, lane r of them its rows r * ROWS .. (r + 1) * ROWS - 1 (rows past
+// dim are zero and stay zero).  Block: R * vdim threads rounded up to whole waves; thread = R *
+// column + r.  The state of a head lies in memory as S transposed and padded, [vdim][R * ROWS].
+template <typename T, int R, int ROWS>
 __global__ __launch_bounds__(1024) void gated_delta_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, const T* __restrict__ proj, int64_t proj_stride, int col_b,
     int col_a, int col_g, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
@@ -100,11 +119,11 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
     const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ out, int64_t out_stride, int heads,
     int kv_heads, int dim, int vdim, float eps, int num_slots) {
   constexpr bool WIDE = sizeof(T) == 4;
+  constexpr int PAD = R * ROWS;  // rows of S as kept: dim rounded up
   extern __shared__ __align__(16) unsigned char lds_bytes[];
-  const int dim4 = (dim + 3) / 4 * 4;
-  float* q_tile = reinterpret_cast<float*>(lds_bytes);  // [TILE][dim4]
-  float* k_tile = q_tile + DELTA_TILE * dim4;           // [TILE][dim4]
-  float* o_tile = k_tile + DELTA_TILE * dim4;           // [TILE][vdim]
+  float* q_tile = reinterpret_cast<float*>(lds_bytes);  // [TILE][PAD]
+  float* k_tile = q_tile + DELTA_TILE * PAD;            // [TILE][PAD]
+  float* o_tile = k_tile + DELTA_TILE * PAD;            // [TILE][vdim]
   TokenGates* gates = reinterpret_cast<TokenGates*>(o_tile + DELTA_TILE * vdim);  // [TILE]
 
   const int h = blockIdx.x, b = blockIdx.y;
@@ -112,16 +131,18 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
   if (last <= first) return;
   const int slot = slots[b];
   const int tid = threadIdx.x, lane = tid % MI_WAVE, wave = tid / MI_WAVE, n_waves = blockDim.x / MI_WAVE;
-  const int j = tid >> 2, r = tid & 3;
+  const int j = tid / R, r = tid % R;
   const bool owns = j < vdim;
   const int group = heads / kv_heads;
   const int kvh = h / group;
-  const int quads = (dim + 3) / 4;
   float* mine = state + (int64_t)((slot < 0 || slot >= num_slots) ? num_slots : slot) * state_stride +
-                (int64_t)h * quads * vdim * 4;
+                ((int64_t)h * vdim + (owns ? j : 0)) * PAD + r * ROWS;
   float s[ROWS];
 #pragma unroll
-  for (int ii = 0; ii < ROWS; ++ii) s[ii] = (owns && ii < quads) ? mine[((int64_t)ii * vdim + j) * 4 + r] : 0.f;
+  for (int ii = 0; ii < ROWS; ii += 4) {
+    const float4 four = owns ? *reinterpret_cast<const float4*>(mine + ii) : make_float4(0.f, 0.f, 0.f, 0.f);
+    s[ii] = four.x, s[ii + 1] = four.y, s[ii + 2] = four.z, s[ii + 3] = four.w;
+  }
 
   const int q_col = kvh * dim, k_col = kv_heads * dim + kvh * dim, v_col = 2 * kv_heads * dim + h * vdim;
   const float rate = expf(a_log[h]);
@@ -136,11 +157,11 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
       const T* row = qkv + (int64_t)(t0 + i) * qkv_stride;
       float qq = 0.f, kk = 0.f;
       double qq_wide = 0.0, kk_wide = 0.0;
-      for (int d = lane; d < dim4; d += MI_WAVE) {
+      for (int d = lane; d < PAD; d += MI_WAVE) {
         const float qv = d < dim ? to_f32(row[q_col + d]) : 0.f;
         const float kv = d < dim ? to_f32(row[k_col + d]) : 0.f;
-        q_tile[i * dim4 + d] = qv;
-        k_tile[i * dim4 + d] = kv;
+        q_tile[i * PAD + d] = qv;
+        k_tile[i * PAD + d] = kv;
         if constexpr (WIDE) {
           qq_wide += (double)qv * qv;
           kk_wide += (double)kv * kv;
@@ -162,9 +183,9 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
         q_inv = rsqrtf(wave_sum(qq) + 1e-6f) * q_scale;
         k_inv = rsqrtf(wave_sum(kk) + 1e-6f);
       }
-      for (int d = lane; d < dim4; d += MI_WAVE) {  // (a lane rescales what it wrote itself)
-        q_tile[i * dim4 + d] *= q_inv;
-        k_tile[i * dim4 + d] *= k_inv;
+      for (int d = lane; d < PAD; d += MI_WAVE) {  // (a lane rescales what it wrote itself)
+        q_tile[i * PAD + d] *= q_inv;
+        k_tile[i * PAD + d] *= k_inv;
       }
       if (lane == 0) {
         const T* p = proj + (int64_t)(t0 + i) * proj_stride;
@@ -185,35 +206,38 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
       }
     }
     __syncthreads();
-    // -- the recurrence over the tile's tokens: no barrier, the four lanes of a column meet by exchange
+    // -- the recurrence over the tile's tokens: no barrier, the lanes of a column meet by register moves
     float v_next = owns ? to_f32(qkv[(int64_t)t0 * qkv_stride + v_col + j]) : 0.f;
     for (int i = 0; i < nt; ++i) {
       const float v = v_next;
       if (i + 1 < nt) v_next = owns ? to_f32(qkv[(int64_t)(t0 + i + 1) * qkv_stride + v_col + j]) : 0.f;
       const TokenGates gt = gates[i];
-      const float* kt = k_tile + i * dim4 + r;
-      const float* qt = q_tile + i * dim4 + r;
+      const float4* kt = reinterpret_cast<const float4*>(k_tile + i * PAD + r * ROWS);
+      const float4* qt = reinterpret_cast<const float4*>(q_tile + i * PAD + r * ROWS);
+      float kr[ROWS];
       float seen = 0.f;
 #pragma unroll
-      for (int ii = 0; ii < ROWS; ++ii) {
-        if (ii < quads) {
-          s[ii] *= gt.decay;
-          seen = fmaf(s[ii], kt[4 * ii], seen);
-        }
+      for (int ii = 0; ii < ROWS; ii += 4) {
+        const float4 four = kt[ii / 4];
+        kr[ii] = four.x, kr[ii + 1] = four.y, kr[ii + 2] = four.z, kr[ii + 3] = four.w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) seen = fmaf(s[ii + e], kr[ii + e], seen);
       }
-      seen += __shfl_xor(seen, 1, MI_WAVE);
-      seen += __shfl_xor(seen, 2, MI_WAVE);
+      // (S^T k of the decayed state is the decay times S^T k of the old one)
+      seen = lanes_sum<R>(seen) * gt.decay;
       const float u = gt.write * (v - seen);
       float read = 0.f;
 #pragma unroll
-      for (int ii = 0; ii < ROWS; ++ii) {
-        if (ii < quads) {
-          s[ii] = fmaf(kt[4 * ii], u, s[ii]);
-          read = fmaf(s[ii], qt[4 * ii], read);
+      for (int ii = 0; ii < ROWS; ii += 4) {
+        const float4 four = qt[ii / 4];
+        const float qr[4] = {four.x, four.y, four.z, four.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[ii + e] = fmaf(kr[ii + e], u, s[ii + e] * gt.decay);
+          read = fmaf(s[ii + e], qr[e], read);
         }
       }
-      read += __shfl_xor(read, 1, MI_WAVE);
-      read += __shfl_xor(read, 2, MI_WAVE);
+      read = lanes_sum<R>(read);
       if (owns && r == 0) o_tile[i * vdim + j] = read;
     }
     __syncthreads();
@@ -251,9 +275,16 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
   }
   if (owns) {
 #pragma unroll
-    for (int ii = 0; ii < ROWS; ++ii)
-      if (ii < quads) mine[((int64_t)ii * vdim + j) * 4 + r] = s[ii];
+    for (int ii = 0; ii < ROWS; ii += 4) *reinterpret_cast<float4*>(mine + ii) = make_float4(s[ii], s[ii + 1], s[ii + 2], s[ii + 3]);
   }
+}
+
+// How a head's state is kept for these sizes: R lanes a column (as many as fit a block of 1024
+// threads, 16 at most), ROWS rows a lane (4, 16 or 64: the next of them that holds dim / R).
+static void delta_layout(int dim, int vdim, int* lanes, int* rows) {
+  *lanes = vdim <= 64 ? 16 : (vdim <= 128 ? 8 : 4);
+  const int need = ceil_div(dim, *lanes);
+  *rows = need <= 4 ? 4 : (need <= 16 ? 16 : 64);
 }
 
 }  // namespace
@@ -301,20 +332,32 @@ extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const f
 
 // qkv: the convolved q | k | v [tokens, 2 * kv_heads * dim + heads * vdim]; proj: the row that
 // holds the write gates' (col_b), the decays' (col_a, heads columns each) and the output gates'
-// (col_g, heads * vdim columns) projections; state float32 [slots + 1, heads * ceil(dim/4) * vdim * 4].
+// (col_g, heads * vdim columns) projections; state float32 [slots + 1, heads * vdim * dim_pad], dim_pad what
+// mi_gated_delta_rows says for these sizes.
+extern "C" int mi_gated_delta_rows(int dim, int vdim) {
+  int lanes = 0, rows = 0;
+  delta_layout(dim, vdim, &lanes, &rows);
+  return lanes * rows;
+}
+
 extern "C" int mi_gated_delta(int dtype, const void* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
                               int col_b, int col_a, int col_g, const float* a_log, const float* dt_bias,
                               const float* norm_weight, float* state, int64_t state_stride, const int* cu,
                               const int* slots, void* out, int64_t out_stride, int num_requests, int heads,
-                              int kv_heads, int dim, int vdim, float eps, int num_slots, hipStream_t stream) {
+                              int kv_heads, int dim, int vdim, int dim_pad, float eps, int num_slots, hipStream_t stream) {
   MI_REQUIRE(num_requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
              "gated_delta: bad sizes requests=%d heads=%d kv_heads=%d", num_requests, heads, kv_heads);
   MI_REQUIRE(dim > 0 && dim <= 256, "gated_delta: dim=%d must be 1..256", dim);
   MI_REQUIRE(vdim > 0 && vdim <= 256, "gated_delta: vdim=%d must be 1..256", vdim);
-  const int quads = (dim + 3) / 4;
-  MI_REQUIRE(qkv_stride >= 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim && out_stride >= (int64_t)heads * vdim &&
-                 state_stride >= (int64_t)heads * quads * vdim * 4,
+  int lanes = 0, rows = 0;
+  delta_layout(dim, vdim, &lanes, &rows);
+  const int pad = lanes * rows;
+  MI_REQUIRE(qkv_stride >= 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim && out_stride >= (int64_t)heads * vdim,
              "gated_delta: row strides shorter than a row");
+  MI_REQUIRE(dim_pad == pad && state_stride >= (int64_t)heads * vdim * pad && state_stride % 4 == 0 &&
+                 (uintptr_t)state % 16 == 0,
+             "gated_delta: heads of %d x %d keep their state as [vdim][%d] float32 on 16-byte boundaries, the caller has [vdim][%d]",
+             dim, vdim, pad, dim_pad);
   MI_REQUIRE(col_b >= 0 && col_a >= 0 && col_g >= 0 && proj_stride >= col_b + heads && proj_stride >= col_a + heads &&
                  proj_stride >= col_g + (int64_t)heads * vdim,
              "gated_delta: the gates' columns lie outside a row of the projections");
@@ -322,21 +365,24 @@ extern "C" int mi_gated_delta(int dtype, const void* qkv, int64_t qkv_stride, co
   MI_REQUIRE(num_slots >= 1 && num_requests <= 65535, "gated_delta: bad slot or request count");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "gated_delta: unknown dtype %d", dtype);
   if (num_requests == 0) return MI_OK;
-  const int threads = ceil_div(4 * vdim, MI_WAVE) * MI_WAVE;
-  const int dim4 = quads * 4;
-  const size_t lds = sizeof(float) * DELTA_TILE * (2 * dim4 + vdim) + sizeof(TokenGates) * DELTA_TILE;
+  const int threads = ceil_div(lanes * vdim, MI_WAVE) * MI_WAVE;
+  const size_t lds = sizeof(float) * DELTA_TILE * (2 * pad + vdim) + sizeof(TokenGates) * DELTA_TILE;
   dim3 grid(heads, num_requests);
-#define MI_DELTA_LAUNCH(T, ROWS)                                                                                       \
-  gated_delta_kernel<T, ROWS><<<grid, threads, lds, stream>>>(                                                         \
+#define MI_DELTA_LAUNCH(T, RR, ROWS)                                                                                   \
+  gated_delta_kernel<T, RR, ROWS><<<grid, threads, lds, stream>>>(                                                     \
       (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, col_b, col_a, col_g, a_log, dt_bias, norm_weight, state, \
       state_stride, cu, slots, (T*)out, out_stride, heads, kv_heads, dim, vdim, eps, num_slots)
-#define MI_DELTA_ROWS(T)                         \
-  if (quads <= 8) MI_DELTA_LAUNCH(T, 8);         \
-  else if (quads <= 16) MI_DELTA_LAUNCH(T, 16);  \
-  else if (quads <= 32) MI_DELTA_LAUNCH(T, 32);  \
-  else MI_DELTA_LAUNCH(T, 64)
-  if (dtype == MI_F32) { MI_DELTA_ROWS(float); }
-  else { MI_DELTA_ROWS(bf16_t); }
+#define MI_DELTA_ROWS(T, RR)                      \
+  if (rows == 4) MI_DELTA_LAUNCH(T, RR, 4);       \
+  else if (rows == 16) MI_DELTA_LAUNCH(T, RR, 16); \
+  else MI_DELTA_LAUNCH(T, RR, 64)
+#define MI_DELTA_LANES(T)                   \
+  if (lanes == 16) { MI_DELTA_ROWS(T, 16); } \
+  else if (lanes == 8) { MI_DELTA_ROWS(T, 8); } \
+  else { MI_DELTA_ROWS(T, 4); }
+  if (dtype == MI_F32) { MI_DELTA_LANES(float) }
+  else { MI_DELTA_LANES(bf16_t) }
+#undef MI_DELTA_LANES
 #undef MI_DELTA_ROWS
 #undef MI_DELTA_LAUNCH
   MI_CHECK_LAUNCH("gated_delta");

@@ -917,7 +917,8 @@ def paged_attention(
     `v_head_dim`: value rows of another width than the keys' (the result is then
     [T, q_heads*v_head_dim]); with `v_pages=None` a value row is the first `v_head_dim` entries
     of its key row.  `sink_logit`: the softmax's denominator gets one more term
-    exp(sink_logit), a sink that carries no value.  These run the plain kernel.
+    exp(sink_logit), a sink that carries no value (both attention kernels know it; uncombined
+    `AttentionPieces` do not).  Values of a width of their own run the plain kernel.
 
     `slopes` (float32 [q_heads], optional): the score of head h for the key at position j
     seen from position p gets `slopes[h] * (j - p)` added before the softmax.  Only the
@@ -937,7 +938,7 @@ def paged_attention(
     bfloat16 caches with transposed values run on the matrix cores; everything else
     (float32, other head or page sizes) runs the plain kernel.
     """
-    if v_pages is None or sink_logit is not None or (v_head_dim is not None and v_head_dim != head_dim):
+    if v_pages is None or (v_head_dim is not None and v_head_dim != head_dim) or (sink_logit is not None and not v_transposed):
         return _paged_attention_general(
             q, k_pages, v_pages, block_table, token_request, positions, q_heads=q_heads, kv_heads=kv_heads,
             head_dim=head_dim, v_head_dim=head_dim if v_head_dim is None else int(v_head_dim), scale=scale,
@@ -1016,7 +1017,7 @@ def paged_attention(
                 _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
                 _ptr(cu_seqlens_q), _ptr(positions), num_requests, tokens, num_tiles, _ptr(out), out.stride(0),
                 _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads, head_dim, page_size, num_pages, float(scale),
-                int(window or 0), splits, shape, 0, 0, 1, _stream(),
+                int(window or 0), splits, shape, 0, 0, 1, int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
             )
         )
         return out
@@ -1059,7 +1060,7 @@ def paged_attention(
                     num_tiles, _ptr(out), out.stride(0), _ptr(part_acc), _ptr(part_ml), q_heads, kv_heads,
                     head_dim, page_size, num_pages, float(scale), int(window or 0), splits,
                     shape, int(one_tile_per_request), first_token,
-                    0 if (leave_pieces and splits > 1) else 1, _stream(),
+                    0 if (leave_pieces and splits > 1) else 1, int(sink_logit is not None), float(sink_logit or 0.0), _stream(),
                 )
             )
             if leave_pieces and splits > 1:
@@ -1077,7 +1078,7 @@ def paged_attention(
             run(0, leading_single)
             run(leading_single, num_requests)
         else:
-            pieces = run(0, num_requests, leave_pieces=not combine and leading_single == num_requests)
+            pieces = run(0, num_requests, leave_pieces=not combine and sink_logit is None and leading_single == num_requests)
             if pieces is not None:
                 return pieces
         return out
@@ -1587,10 +1588,14 @@ def short_conv(
     return y
 
 
-def delta_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int, int]:
-    """How `gated_delta` lays a request's state out: per head [ceil(dim/4)][vdim][4], element
-    (i, j) of S at [i // 4][j][i % 4]."""
-    return (heads, -(-dim // 4), vdim, 4)
+def delta_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int]:
+    """How `gated_delta` lays a request's state out: per head S transposed, [vdim][padded dim].
+    A column is kept by 16, 8 or 4 neighbouring lanes (as many as fit a block of 1,024 threads),
+    each holding 4, 16 or 64 rows: the padded dim is their product (the kernel checks it)."""
+    lanes = 16 if vdim <= 64 else (8 if vdim <= 128 else 4)
+    need = -(-dim // lanes)
+    rows = 4 if need <= 4 else (16 if need <= 16 else 64)
+    return (heads, vdim, lanes * rows)
 
 
 def gated_delta(
@@ -1620,7 +1625,7 @@ def gated_delta(
     if a_log.numel() != heads or dt_bias.numel() != heads or norm_weight.numel() != vdim:
         raise KernelShapeError("gated_delta: one decay rate and one step bias per head, one norm weight per value column")
     shape = delta_state_shape(heads, dim, vdim)
-    if state.dim() != 5 or tuple(state.shape[1:]) != shape or state.shape[0] < 2 or not state[0].is_contiguous():
+    if state.dim() != 4 or tuple(state.shape[1:]) != shape or state.shape[0] < 2 or not state[0].is_contiguous():
         raise KernelShapeError(f"gated_delta: the state is float32 [slots + 1, {shape}] with packed slots, got {tuple(state.shape)}")
     requests = slots.numel()
     if cu_seqlens.numel() != requests + 1:
@@ -1630,7 +1635,7 @@ def gated_delta(
         library.load().mi_gated_delta(
             _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(col_b), int(col_a), int(col_g),
             _ptr(a_log), _ptr(dt_bias), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(slots),
-            _ptr(out), out.stride(0), requests, heads, kv_heads, dim, vdim, float(eps), state.shape[0] - 1, _stream(),
+            _ptr(out), out.stride(0), requests, heads, kv_heads, dim, vdim, shape[2], float(eps), state.shape[0] - 1, _stream(),
         )
     )
     return out
@@ -1678,8 +1683,9 @@ def latent_prepare(
 def linear_per_head(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
     """`out[:, h, :] = x[:, h, :] @ weight[h].T` for every head h: x [T, heads, K], weight
     [heads, N, K], out [T, heads, N]; x and out may be views into wider rows (unit inner
-    stride).  float32: the true-float32 product, head by head; few bfloat16 rows: the
-    weight-streaming product, head by head; else one batched product of the vendor library."""
+    stride).  float32: the true-float32 product, head by head; bfloat16: one batched product of
+    the vendor library (the weight-streaming product has no batched form; head by head it costs a
+    launch a head, which at few rows is all a step's time)."""
     _need_cuda(x, weight, out)
     if x.dim() != 3 or weight.dim() != 3 or out.dim() != 3 or x.stride(2) != 1 or out.stride(2) != 1 or weight.stride(2) != 1:
         raise KernelShapeError("linear_per_head: x [T, heads, K], weight [heads, N, K], out [T, heads, N], unit inner strides")
@@ -1694,11 +1700,6 @@ def linear_per_head(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) ->
         for h in range(heads):
             library.check(lib.mi_gemm_f32(_ptr(x[:, h]), x.stride(0), _ptr(weight[h]), weight.stride(1), _ptr(out[:, h]),
                                           out.stride(0), tokens, n, k, _stream()))
-        return
-    if skinny_gemm_takes(tokens, k, x.stride(0), weight.stride(1)) and x.stride(1) % 8 == 0 and weight.stride(0) % 8 == 0:
-        for h in range(heads):
-            library.check(lib.mi_gemm_skinny_bf16(_ptr(x[:, h]), x.stride(0), _ptr(weight[h]), weight.stride(1),
-                                                  _ptr(out[:, h]), out.stride(0), tokens, n, k, _stream()))
         return
     torch.bmm(x.transpose(0, 1), weight.transpose(1, 2), out=out.transpose(0, 1))
 

@@ -72,8 +72,8 @@ class GQAttention(Mixer):
         if self.v_head_dim <= 0 or self.v_head_dim % ops.ATTENTION_HEAD_DIM_STEP != 0:
             raise ValueError(f"v_head_dim={self.v_head_dim}: the attention kernels take even value head sizes")
         self.sink_logit = None if sink_logit is None else float(sink_logit)
-        # what the matrix-core kernel and the fused few-row kernels know: no sink, values as wide as keys
-        self._plain_softmax = self.sink_logit is None and self.v_head_dim == head_dim
+        # what the matrix-core kernel and the fused few-row kernels take: values as wide as keys
+        self._same_widths = self.v_head_dim == head_dim
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
@@ -105,7 +105,7 @@ class GQAttention(Mixer):
         layout = self.position.rotary_layout() if self.position is not None else None
         return (
             self.dtype == torch.bfloat16
-            and self._plain_softmax
+            and self._same_widths
             and layout == (self.head_dim, False)
             and self.head_dim % 32 == 0
             and ops.scaled_rows_product_takes(rows, self.qkv.weight, self.hidden_size)
@@ -115,7 +115,7 @@ class GQAttention(Mixer):
         # values lie transposed inside a page where the matrix-core kernel will read them
         # (that kernel knows no score bias: such layers keep the plain layout and kernel)
         transposed = (
-            self.slopes is None and self._plain_softmax
+            self.slopes is None and self._same_widths
             and ops.mfma_attention_supported(self.dtype, self.head_dim, page_size)
         )
         v_head_dim = None if self.v_head_dim == self.head_dim else self.v_head_dim
@@ -132,11 +132,11 @@ class GQAttention(Mixer):
         rotary = self.position.rotary(ctx) if self.position is not None else None
         if isinstance(x, ops.ScaledRows) and not (
             rotary is not None
-            and self._plain_softmax
+            and self._same_widths
             and ops.qkv_rope_write_takes(x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved)
         ):
             x = x.finish()  # rows but for their norm factors, and no kernel here that applies them
-        if rotary is not None and self._plain_softmax and ops.qkv_rope_write_takes(
+        if rotary is not None and self._same_widths and ops.qkv_rope_write_takes(
             x, self.qkv.weight, self.head_dim, rotary.rotary_dim, rotary.interleaved
         ):
             # few rows (decode): projection, rotation and cache write are one kernel
@@ -186,7 +186,7 @@ class GQAttention(Mixer):
         At the smallest batches the key ranges may come back uncombined, for the output
         projection to combine on its way (one launch less a layer)."""
         few = (
-            queries.dtype == torch.bfloat16 and self._plain_softmax
+            queries.dtype == torch.bfloat16 and self._same_widths and self.sink_logit is None
             and ops.attention_pieces_pay(ctx.num_tokens, self.num_heads, self.head_dim)
         )
         return ops.paged_attention(

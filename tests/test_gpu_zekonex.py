@@ -159,7 +159,8 @@ def paged(rows: np.ndarray, page_size: int, order: list[int], dtype) -> torch.Te
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads, kv_heads, dim, vdim, page", [(4, 2, 16, 24, 8), (3, 3, 10, 6, 4), (8, 1, 64, 64, 16), (5, 1, 130, 66, 16)])
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim, page", [(4, 2, 16, 24, 8), (3, 3, 10, 6, 4), (8, 1, 64, 64, 16), (5, 1, 130, 66, 16),
+                                                               (8, 2, 128, 128, 16), (4, 4, 32, 32, 32)])
 def test_attention_with_a_sink_and_values_of_another_width(dtype, heads, kv_heads, dim, vdim, page):
     """One request of 333 keys in scattered pages, queries at its last 5 positions.  Head 0's
     last query is made to single out key 3, far back; head 1's scores are all far below the
@@ -201,6 +202,18 @@ def test_attention_with_a_sink_and_values_of_another_width(dtype, heads, kv_head
                 sunk = 1.0 / (1.0 + e.sum())
     np.testing.assert_allclose(got, want, rtol=0, atol=tolerance(dtype, 4))
     assert weight_on_3 > 0.9  # the far key is what the answer is made of
+    if ops.mfma_attention_supported(TORCH[dtype], dim, page) and vdim == dim:
+        # the matrix-core kernel (values transposed inside a page) knows the sink too: the queries as a
+        # prompt's last portion, and the last one alone as a decoded token (keys cut into ranges)
+        v_t = paged(v, page, order, dtype).transpose(2, 3).contiguous()
+        for rows in (slice(0, queries_n), slice(queries_n - 1, queries_n)):
+            n = rows.stop - rows.start
+            fast = ops.paged_attention(
+                dev(q[rows].reshape(n, -1), TORCH[dtype]), paged(k, page, order, dtype), v_t, ints(order).view(1, -1), ints([0] * n),
+                ints(positions[rows]), ints([0, n]), [0, n], q_heads=heads, kv_heads=kv_heads, head_dim=dim, scale=scale,
+                window=None, max_seq_len=keys_n, v_transposed=True, sink_logit=0.0,
+            ).float().cpu().numpy().reshape(n, heads, vdim)
+            np.testing.assert_allclose(fast, want[rows], rtol=0, atol=tolerance(dtype, 4))
     if heads > 1:
         assert sunk > 0.99 and np.abs(want[:, 1]).max() < 0.05 < np.abs(vq).mean()  # a sink left out would show
 

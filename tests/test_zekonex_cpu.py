@@ -43,7 +43,7 @@ def test_every_pass_of_a_loop_has_caches_and_state_of_its_own():
     needs = model_of(cfg).cache_needs(block)
     assert len(needs) == 8 and all(need is not None for need in needs)
     first = needs[0].state
-    assert first["recurrent"].shape == (4, 3, 20, 4) and first["recurrent"].dtype == torch.float32
+    assert first["recurrent"].shape == (4, 20, 64) and first["recurrent"].dtype == torch.float32
     assert first["tail"].shape == (2, 2 * 4 * 12 + 4 * 20) and first["tail"].dtype == torch.bfloat16
     assert needs[2].state == first and needs[4].state == first
     pages = needs[1].pages  # attention: keys of 16, values of 24
