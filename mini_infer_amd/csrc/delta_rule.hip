@@ -14,10 +14,10 @@
 //                     per column and silu(g).
 //
 // The state of a head lies in memory transposed and padded, [vdim][dim_pad].  Column j of S is
-// kept by R neighbouring lanes (4, 8 or 16), each holding a run of its rows: a token costs a lane
-// dim/R multiply-adds per pass and the partial sums meet through register moves between the
-// lanes, with no barrier inside a tile of tokens.  Columns are independent of one another, so a
-// head's work spreads over R * vdim threads however short the step.
+// kept by 16 neighbouring lanes, each holding a run of its rows: a token costs a lane dim/16
+// multiply-adds per pass and the partial sums meet through register moves between the lanes,
+// with no barrier inside a tile of tokens.  Columns are independent of one another, so a head's
+// work spreads over 16 * vdim threads however short the step.
 // Everything that enters the recurrence is float32 (the projections and the convolution's
 // outputs are read in the element type); in the 32-bit engine the scalar gates, the unit norms
 // and the read-out's norm are evaluated in 64-bit and rounded once.
@@ -25,7 +25,6 @@
 
 #include <math.h>
 
-#define DELTA_TILE 16      // tokens whose q, k, gates are prepared together
 #define DELTA_MAX_TAPS 16
 
 namespace {
@@ -108,30 +107,46 @@ __device__ __forceinline__ float lanes_sum(float v) {
   return v;
 }
 
-// R lanes keep a column of S, lane r of them its rows r * ROWS .. (r + 1) * ROWS - 1 (rows past
-// dim are zero and stay zero).  Block: R * vdim threads rounded up to whole waves; thread = R *
-// column + r.  The state of a head lies in memory as S transposed and padded, [vdim][R * ROWS].
-template <typename T, int R, int ROWS>
-__global__ __launch_bounds__(1024) void gated_delta_kernel(
+// 16 lanes keep a column of S, lane r of them its rows r * ROWS .. (r + 1) * ROWS - 1 (rows past
+// dim are zero and stay zero).  The columns of S do not meet in the recurrence, so a head's
+// columns are shared out among blocks: 256 threads keep 16 columns; thread = 16 * column + r.
+// The state of a head lies in memory as S transposed and padded, [vdim][16 * ROWS].  The read-outs
+// leave as float32 [tokens, heads * vdim]; their norm over a head's columns is the next kernel's.
+//
+// Tokens are taken 32 at a time.  A tile's rows are asked of memory while the tile before it is
+// worked on (they wait in registers); then 8 lanes a token make q and k unit vectors and put
+// them into LDS with the tile's values and gates, all 32 tokens at once; then the recurrence
+// walks the tile with LDS reads only, each token's operands read while the one before it is
+// worked on.  A step of the recurrence is 4 * ROWS multiply-adds a lane and two sums over 16
+// lanes by register moves.
+template <typename T, int ROWS>
+__global__ __launch_bounds__(256) void gated_delta_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, const T* __restrict__ proj, int64_t proj_stride, int col_b,
-    int col_a, int col_g, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
-    const float* __restrict__ norm_weight, float* __restrict__ state, int64_t state_stride,
-    const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ out, int64_t out_stride, int heads,
-    int kv_heads, int dim, int vdim, float eps, int num_slots) {
+    int col_a, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
+    int64_t state_stride, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ readout,
+    int heads, int kv_heads, int dim, int vdim, int chunks, int num_slots) {
   constexpr bool WIDE = sizeof(T) == 4;
-  constexpr int PAD = R * ROWS;  // rows of S as kept: dim rounded up
-  extern __shared__ __align__(16) unsigned char lds_bytes[];
-  float* q_tile = reinterpret_cast<float*>(lds_bytes);  // [TILE][PAD]
-  float* k_tile = q_tile + DELTA_TILE * PAD;            // [TILE][PAD]
-  float* o_tile = k_tile + DELTA_TILE * PAD;            // [TILE][vdim]
-  TokenGates* gates = reinterpret_cast<TokenGates*>(o_tile + DELTA_TILE * vdim);  // [TILE]
+  constexpr int R = 16;            // lanes a column
+  constexpr int PAD = R * ROWS;    // rows of S as kept: dim rounded up
+  constexpr int COLS = 256 / R;    // columns of S this block keeps
+  constexpr int TILE = 32;         // tokens prepared together
+  constexpr int GROUP = 8;         // lanes that prepare one token
+  constexpr int EACH = PAD / GROUP;  // entries of a token's q (and k) row a lane prepares: two runs of ROWS
+  // (a lane's run of ROWS entries is followed by 4 unused ones: the runs that a 16-byte read of
+  // all lanes touches then lie in different banks)
+  constexpr int RUN = ROWS + 4;
+  constexpr int LPAD = R * RUN;
+  __shared__ __align__(16) float q_tile[TILE * LPAD];
+  __shared__ __align__(16) float k_tile[TILE * LPAD];
+  __shared__ float v_tile[TILE * COLS];
+  __shared__ TokenGates gates[TILE];
 
-  const int h = blockIdx.x, b = blockIdx.y;
+  const int h = blockIdx.x / chunks, chunk = blockIdx.x % chunks, b = blockIdx.y;
   const int first = cu[b], last = cu[b + 1];
   if (last <= first) return;
   const int slot = slots[b];
-  const int tid = threadIdx.x, lane = tid % MI_WAVE, wave = tid / MI_WAVE, n_waves = blockDim.x / MI_WAVE;
-  const int j = tid / R, r = tid % R;
+  const int tid = threadIdx.x;
+  const int j = chunk * COLS + tid / R, r = tid % R;
   const bool owns = j < vdim;
   const int group = heads / kv_heads;
   const int kvh = h / group;
@@ -144,133 +159,138 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
     s[ii] = four.x, s[ii + 1] = four.y, s[ii + 2] = four.z, s[ii + 3] = four.w;
   }
 
-  const int q_col = kvh * dim, k_col = kv_heads * dim + kvh * dim, v_col = 2 * kv_heads * dim + h * vdim;
+  const int q_col = kvh * dim, k_col = kv_heads * dim + kvh * dim, v_col = 2 * kv_heads * dim + h * vdim + chunk * COLS;
+  const int my_cols = min(COLS, vdim - chunk * COLS);
   const float rate = expf(a_log[h]);
   const double rate_wide = exp((double)a_log[h]);
   const float q_scale = 1.0f / sqrtf((float)dim);
+  const float bias = dt_bias[h];
 
-  for (int t0 = first; t0 < last; t0 += DELTA_TILE) {
-    const int nt = min(DELTA_TILE, last - t0);
-    __syncthreads();  // the last tile's read-outs have been written out
-    // -- q and k of the tile's tokens: unit vectors (float32 from here on); a wave takes a token
-    for (int i = wave; i < nt; i += n_waves) {
-      const T* row = qkv + (int64_t)(t0 + i) * qkv_stride;
-      float qq = 0.f, kk = 0.f;
-      double qq_wide = 0.0, kk_wide = 0.0;
-      for (int d = lane; d < PAD; d += MI_WAVE) {
-        const float qv = d < dim ? to_f32(row[q_col + d]) : 0.f;
-        const float kv = d < dim ? to_f32(row[k_col + d]) : 0.f;
-        q_tile[i * PAD + d] = qv;
-        k_tile[i * PAD + d] = kv;
-        if constexpr (WIDE) {
-          qq_wide += (double)qv * qv;
-          kk_wide += (double)kv * kv;
-        } else {
-          qq += qv * qv;
-          kk += kv * kv;
-        }
-      }
+  // what this thread prepares of a tile: token `mine_token` (8 lanes a token), entries
+  // sub * EACH .. of its q and k rows; and two of the tile's values
+  const int mine_token = tid / GROUP, sub = tid % GROUP;
+  float q_raw[EACH], k_raw[EACH], v_raw[2], b_raw = 0.f, a_raw = 0.f;
+  auto ask = [&](int t0, int nt) {
+    const bool live = mine_token < nt;
+    const T* row = qkv + (int64_t)(t0 + (live ? mine_token : 0)) * qkv_stride;
+#pragma unroll
+    for (int e = 0; e < EACH; ++e) {
+      const int d = sub * EACH + e;
+      q_raw[e] = (live && d < dim) ? to_f32(row[q_col + d]) : 0.f;
+      k_raw[e] = (live && d < dim) ? to_f32(row[k_col + d]) : 0.f;
+    }
+    if (sub == 0) {
+      const T* p = proj + (int64_t)(t0 + (live ? mine_token : 0)) * proj_stride;
+      b_raw = to_f32(p[col_b + h]);
+      a_raw = to_f32(p[col_a + h]);
+    }
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int e = tid + n * 256, i = e / COLS, c = e % COLS;
+      v_raw[n] = (i < nt && c < my_cols) ? to_f32(qkv[(int64_t)(t0 + i) * qkv_stride + v_col + c]) : 0.f;
+    }
+  };
+  ask(first, min(TILE, last - first));
+
+  for (int t0 = first; t0 < last; t0 += TILE) {
+    const int nt = min(TILE, last - t0);
+    __syncthreads();  // the last tile's steps have read what is overwritten now
+    {
       float q_inv, k_inv;
       if constexpr (WIDE) {
+        double qq = 0.0, kk = 0.0;
 #pragma unroll
-        for (int off = MI_WAVE / 2; off > 0; off >>= 1) {
-          qq_wide += __shfl_xor(qq_wide, off, MI_WAVE);
-          kk_wide += __shfl_xor(kk_wide, off, MI_WAVE);
+        for (int e = 0; e < EACH; ++e) {
+          qq += (double)q_raw[e] * q_raw[e];
+          kk += (double)k_raw[e] * k_raw[e];
         }
-        q_inv = (float)(1.0 / sqrt((qq_wide + 1e-6) * (double)dim));
-        k_inv = (float)(1.0 / sqrt(kk_wide + 1e-6));
+#pragma unroll
+        for (int off = 1; off < GROUP; off <<= 1) {
+          qq += __shfl_xor(qq, off, MI_WAVE);
+          kk += __shfl_xor(kk, off, MI_WAVE);
+        }
+        q_inv = (float)(1.0 / sqrt((qq + 1e-6) * (double)dim));
+        k_inv = (float)(1.0 / sqrt(kk + 1e-6));
       } else {
-        q_inv = rsqrtf(wave_sum(qq) + 1e-6f) * q_scale;
-        k_inv = rsqrtf(wave_sum(kk) + 1e-6f);
+        float qq = 0.f, kk = 0.f;
+#pragma unroll
+        for (int e = 0; e < EACH; ++e) {
+          qq = fmaf(q_raw[e], q_raw[e], qq);
+          kk = fmaf(k_raw[e], k_raw[e], kk);
+        }
+        q_inv = rsqrtf(lanes_sum<GROUP>(qq) + 1e-6f) * q_scale;
+        k_inv = rsqrtf(lanes_sum<GROUP>(kk) + 1e-6f);
       }
-      for (int d = lane; d < PAD; d += MI_WAVE) {  // (a lane rescales what it wrote itself)
-        q_tile[i * PAD + d] *= q_inv;
-        k_tile[i * PAD + d] *= k_inv;
+      // (a lane's entries are two runs of ROWS: runs 2 * sub and 2 * sub + 1 of the token's row)
+      float* q_at = q_tile + mine_token * LPAD + 2 * sub * RUN;
+      float* k_at = k_tile + mine_token * LPAD + 2 * sub * RUN;
+#pragma unroll
+      for (int e = 0; e < EACH; e += 4) {
+        const int at = e + (e / ROWS) * 4;
+        *reinterpret_cast<float4*>(q_at + at) = make_float4(q_raw[e] * q_inv, q_raw[e + 1] * q_inv, q_raw[e + 2] * q_inv, q_raw[e + 3] * q_inv);
+        *reinterpret_cast<float4*>(k_at + at) = make_float4(k_raw[e] * k_inv, k_raw[e + 1] * k_inv, k_raw[e + 2] * k_inv, k_raw[e + 3] * k_inv);
       }
-      if (lane == 0) {
-        const T* p = proj + (int64_t)(t0 + i) * proj_stride;
-        const float bv = to_f32(p[col_b + h]), av = to_f32(p[col_a + h]);
+      if (sub == 0) {
         TokenGates gt;
         if constexpr (WIDE) {
-          const double z = (double)av + (double)dt_bias[h];
+          const double z = (double)a_raw + (double)bias;
           const double soft = z > 30.0 ? z : log1p(exp(z));
           gt.decay = (float)exp(-rate_wide * soft);
-          gt.write = (float)(1.0 / (1.0 + exp(-(double)bv)));
+          gt.write = (float)(1.0 / (1.0 + exp(-(double)b_raw)));
         } else {
-          const float z = av + dt_bias[h];
+          const float z = a_raw + bias;
           const float soft = z > 20.f ? z : log1pf(expf(z));
           gt.decay = expf(-rate * soft);
-          gt.write = 1.f / (1.f + expf(-bv));
+          gt.write = 1.f / (1.f + expf(-b_raw));
         }
-        gates[i] = gt;
+        gates[mine_token] = gt;
       }
+      v_tile[tid] = v_raw[0];
+      v_tile[tid + 256] = v_raw[1];
     }
     __syncthreads();
+    if (t0 + TILE < last) ask(t0 + TILE, min(TILE, last - t0 - TILE));  // (waits in registers through the steps below)
     // -- the recurrence over the tile's tokens: no barrier, the lanes of a column meet by register moves
-    float v_next = owns ? to_f32(qkv[(int64_t)t0 * qkv_stride + v_col + j]) : 0.f;
-    for (int i = 0; i < nt; ++i) {
-      const float v = v_next;
-      if (i + 1 < nt) v_next = owns ? to_f32(qkv[(int64_t)(t0 + i + 1) * qkv_stride + v_col + j]) : 0.f;
-      const TokenGates gt = gates[i];
-      const float4* kt = reinterpret_cast<const float4*>(k_tile + i * PAD + r * ROWS);
-      const float4* qt = reinterpret_cast<const float4*>(q_tile + i * PAD + r * ROWS);
-      float kr[ROWS];
-      float seen = 0.f;
+    float kr[ROWS], qr[ROWS], k_next[ROWS], q_next[ROWS];
+    float v = 0.f, v_after = 0.f;
+    TokenGates gt = {1.f, 0.f}, gt_after = {1.f, 0.f};
+    auto fetch = [&](int i, float* kd, float* qd, float& vd, TokenGates& gd) {
+      const float4* kt = reinterpret_cast<const float4*>(k_tile + i * LPAD + r * RUN);
+      const float4* qt = reinterpret_cast<const float4*>(q_tile + i * LPAD + r * RUN);
 #pragma unroll
       for (int ii = 0; ii < ROWS; ii += 4) {
-        const float4 four = kt[ii / 4];
-        kr[ii] = four.x, kr[ii + 1] = four.y, kr[ii + 2] = four.z, kr[ii + 3] = four.w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) seen = fmaf(s[ii + e], kr[ii + e], seen);
+        const float4 kf = kt[ii / 4], qf = qt[ii / 4];
+        kd[ii] = kf.x, kd[ii + 1] = kf.y, kd[ii + 2] = kf.z, kd[ii + 3] = kf.w;
+        qd[ii] = qf.x, qd[ii + 1] = qf.y, qd[ii + 2] = qf.z, qd[ii + 3] = qf.w;
       }
-      // (S^T k of the decayed state is the decay times S^T k of the old one)
-      seen = lanes_sum<R>(seen) * gt.decay;
-      const float u = gt.write * (v - seen);
-      float read = 0.f;
+      vd = v_tile[i * COLS + tid / R];
+      gd = gates[i];
+    };
+    fetch(0, k_next, q_next, v_after, gt_after);
+    for (int i = 0; i < nt; ++i) {
 #pragma unroll
-      for (int ii = 0; ii < ROWS; ii += 4) {
-        const float4 four = qt[ii / 4];
-        const float qr[4] = {four.x, four.y, four.z, four.w};
+      for (int ii = 0; ii < ROWS; ++ii) kr[ii] = k_next[ii], qr[ii] = q_next[ii];
+      v = v_after, gt = gt_after;
+      if (i + 1 < nt) fetch(i + 1, k_next, q_next, v_after, gt_after);
+      // (four running sums each: a chain of dependent multiply-adds would be the step's time)
+      float seen4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ii = 0; ii < ROWS; ii += 4)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) seen4[e] = fmaf(s[ii + e], kr[ii + e], seen4[e]);
+      // (S^T k of the decayed state is the decay times S^T k of the old one)
+      const float seen = lanes_sum<R>((seen4[0] + seen4[1]) + (seen4[2] + seen4[3])) * gt.decay;
+      const float u = gt.write * (v - seen);
+      float read4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ii = 0; ii < ROWS; ii += 4)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           s[ii + e] = fmaf(kr[ii + e], u, s[ii + e] * gt.decay);
-          read = fmaf(s[ii + e], qr[e], read);
+          read4[e] = fmaf(s[ii + e], qr[ii + e], read4[e]);
         }
-      }
-      read = lanes_sum<R>(read);
-      if (owns && r == 0) o_tile[i * vdim + j] = read;
-    }
-    __syncthreads();
-    // -- read-outs of the tile: norm over vdim, weight, gate; a wave takes a token
-    for (int i = wave; i < nt; i += n_waves) {
-      float sq = 0.f;
-      double sq_wide = 0.0;
-      for (int d = lane; d < vdim; d += MI_WAVE) {
-        const float o = o_tile[i * vdim + d];
-        if constexpr (WIDE) sq_wide += (double)o * o;
-        else sq += o * o;
-      }
-      float inv;
-      double inv_wide = 0.0;
-      if constexpr (WIDE) {
-#pragma unroll
-        for (int off = MI_WAVE / 2; off > 0; off >>= 1) sq_wide += __shfl_xor(sq_wide, off, MI_WAVE);
-        inv_wide = 1.0 / sqrt(sq_wide / (double)vdim + (double)eps);
-        inv = (float)inv_wide;
-      } else {
-        inv = rsqrtf(wave_sum(sq) / (float)vdim + eps);
-      }
-      const T* p = proj + (int64_t)(t0 + i) * proj_stride + col_g + h * vdim;
-      T* dst = out + (int64_t)(t0 + i) * out_stride + h * vdim;
-      for (int d = lane; d < vdim; d += MI_WAVE) {
-        const float g = to_f32(p[d]);
-        if constexpr (WIDE) {
-          const double gate = (double)g / (1.0 + exp(-(double)g));
-          dst[d] = (float)((double)o_tile[i * vdim + d] * inv_wide * (double)norm_weight[d] * gate);
-        } else {
-          dst[d] = from_f32<T>(o_tile[i * vdim + d] * inv * norm_weight[d] * (g * mi_logistic(g)));
-        }
-      }
+      const float read = lanes_sum<R>((read4[0] + read4[1]) + (read4[2] + read4[3]));
+      if (owns && r == 0) readout[(int64_t)(t0 + i) * heads * vdim + (int64_t)h * vdim + j] = read;
     }
   }
   if (owns) {
@@ -279,12 +299,55 @@ __global__ __launch_bounds__(1024) void gated_delta_kernel(
   }
 }
 
-// How a head's state is kept for these sizes: R lanes a column (as many as fit a block of 1024
-// threads, 16 at most), ROWS rows a lane (4, 16 or 64: the next of them that holds dim / R).
+// The read-outs of a step, head by head: divided by their root mean square over the head's
+// columns, times a weight per column, times silu of the output gate's projection.  A wave a head.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_readout_norm_kernel(const float* __restrict__ readout, const T* __restrict__ proj,
+                                                                 int64_t proj_stride, int col_g,
+                                                                 const float* __restrict__ norm_weight, T* __restrict__ out,
+                                                                 int64_t out_stride, int heads, int vdim, float eps) {
+  constexpr bool WIDE = sizeof(T) == 4;
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x % MI_WAVE;
+  for (int h = blockIdx.y * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE; h < heads; h += gridDim.y * (blockDim.x / MI_WAVE)) {
+    const float* o = readout + ((int64_t)t * heads + h) * vdim;
+    float sq = 0.f;
+    double sq_wide = 0.0;
+    for (int d = lane; d < vdim; d += MI_WAVE) {
+      if constexpr (WIDE) sq_wide += (double)o[d] * o[d];
+      else sq += o[d] * o[d];
+    }
+    float inv;
+    double inv_wide = 0.0;
+    if constexpr (WIDE) {
+#pragma unroll
+      for (int off = MI_WAVE / 2; off > 0; off >>= 1) sq_wide += __shfl_xor(sq_wide, off, MI_WAVE);
+      inv_wide = 1.0 / sqrt(sq_wide / (double)vdim + (double)eps);
+      inv = (float)inv_wide;
+    } else {
+      inv = rsqrtf(wave_sum(sq) / (float)vdim + eps);
+    }
+    const T* p = proj + (int64_t)t * proj_stride + col_g + h * vdim;
+    T* dst = out + (int64_t)t * out_stride + h * vdim;
+    for (int d = lane; d < vdim; d += MI_WAVE) {
+      const float g = to_f32(p[d]);
+      if constexpr (WIDE) {
+        const double gate = (double)g / (1.0 + exp(-(double)g));
+        dst[d] = (float)((double)o[d] * inv_wide * (double)norm_weight[d] * gate);
+      } else {
+        dst[d] = from_f32<T>(o[d] * inv * norm_weight[d] * (g * mi_logistic(g)));
+      }
+    }
+  }
+}
+
+// How a head's state is kept for these sizes: 16 lanes a column, ROWS rows a lane (4, 8 or 16: the
+// next of them that holds dim / 16).
 static void delta_layout(int dim, int vdim, int* lanes, int* rows) {
-  *lanes = vdim <= 64 ? 16 : (vdim <= 128 ? 8 : 4);
-  const int need = ceil_div(dim, *lanes);
-  *rows = need <= 4 ? 4 : (need <= 16 ? 16 : 64);
+  (void)vdim;
+  *lanes = 16;
+  const int need = ceil_div(dim, 16);
+  *rows = need <= 4 ? 4 : (need <= 8 ? 8 : 16);
 }
 
 }  // namespace
@@ -333,7 +396,7 @@ extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const f
 // qkv: the convolved q | k | v [tokens, 2 * kv_heads * dim + heads * vdim]; proj: the row that
 // holds the write gates' (col_b), the decays' (col_a, heads columns each) and the output gates'
 // (col_g, heads * vdim columns) projections; state float32 [slots + 1, heads * vdim * dim_pad], dim_pad what
-// mi_gated_delta_rows says for these sizes.
+// mi_gated_delta_rows says for these sizes; readout: float32 scratch [tokens, heads * vdim].
 extern "C" int mi_gated_delta_rows(int dim, int vdim) {
   int lanes = 0, rows = 0;
   delta_layout(dim, vdim, &lanes, &rows);
@@ -343,7 +406,7 @@ extern "C" int mi_gated_delta_rows(int dim, int vdim) {
 extern "C" int mi_gated_delta(int dtype, const void* qkv, int64_t qkv_stride, const void* proj, int64_t proj_stride,
                               int col_b, int col_a, int col_g, const float* a_log, const float* dt_bias,
                               const float* norm_weight, float* state, int64_t state_stride, const int* cu,
-                              const int* slots, void* out, int64_t out_stride, int num_requests, int heads,
+                              const int* slots, float* readout, void* out, int64_t out_stride, int num_tokens, int num_requests, int heads,
                               int kv_heads, int dim, int vdim, int dim_pad, float eps, int num_slots, hipStream_t stream) {
   MI_REQUIRE(num_requests >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
              "gated_delta: bad sizes requests=%d heads=%d kv_heads=%d", num_requests, heads, kv_heads);
@@ -365,26 +428,32 @@ extern "C" int mi_gated_delta(int dtype, const void* qkv, int64_t qkv_stride, co
   MI_REQUIRE(num_slots >= 1 && num_requests <= 65535, "gated_delta: bad slot or request count");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "gated_delta: unknown dtype %d", dtype);
   if (num_requests == 0) return MI_OK;
-  const int threads = ceil_div(lanes * vdim, MI_WAVE) * MI_WAVE;
-  const size_t lds = sizeof(float) * DELTA_TILE * (2 * pad + vdim) + sizeof(TokenGates) * DELTA_TILE;
-  dim3 grid(heads, num_requests);
-#define MI_DELTA_LAUNCH(T, RR, ROWS)                                                                                   \
-  gated_delta_kernel<T, RR, ROWS><<<grid, threads, lds, stream>>>(                                                     \
-      (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, col_b, col_a, col_g, a_log, dt_bias, norm_weight, state, \
-      state_stride, cu, slots, (T*)out, out_stride, heads, kv_heads, dim, vdim, eps, num_slots)
-#define MI_DELTA_ROWS(T, RR)                      \
-  if (rows == 4) MI_DELTA_LAUNCH(T, RR, 4);       \
-  else if (rows == 16) MI_DELTA_LAUNCH(T, RR, 16); \
-  else MI_DELTA_LAUNCH(T, RR, 64)
-#define MI_DELTA_LANES(T)                   \
-  if (lanes == 16) { MI_DELTA_ROWS(T, 16); } \
-  else if (lanes == 8) { MI_DELTA_ROWS(T, 8); } \
-  else { MI_DELTA_ROWS(T, 4); }
+  MI_REQUIRE(readout != nullptr, "gated_delta: no buffer for the read-outs");
+  const int cols = 256 / lanes, chunks = ceil_div(vdim, cols);
+  MI_REQUIRE((int64_t)heads * chunks <= 2147483647, "gated_delta: too many heads");
+  dim3 grid(heads * chunks, num_requests);
+#define MI_DELTA_LAUNCH(T, ROWS)                                                                                 \
+  gated_delta_kernel<T, ROWS><<<grid, 256, 0, stream>>>(                                                         \
+      (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, col_b, col_a, a_log, dt_bias, state, state_stride, \
+      cu, slots, readout, heads, kv_heads, dim, vdim, chunks, num_slots)
+#define MI_DELTA_LANES(T)                     \
+  if (rows == 4) MI_DELTA_LAUNCH(T, 4);       \
+  else if (rows == 8) MI_DELTA_LAUNCH(T, 8);  \
+  else MI_DELTA_LAUNCH(T, 16);
   if (dtype == MI_F32) { MI_DELTA_LANES(float) }
   else { MI_DELTA_LANES(bf16_t) }
 #undef MI_DELTA_LANES
-#undef MI_DELTA_ROWS
 #undef MI_DELTA_LAUNCH
   MI_CHECK_LAUNCH("gated_delta");
+  if (num_tokens > 0) {
+    dim3 ngrid(num_tokens, min(ceil_div(heads, 4), 64));
+    if (dtype == MI_F32)
+      delta_readout_norm_kernel<float><<<ngrid, 256, 0, stream>>>(readout, (const float*)proj, proj_stride, col_g, norm_weight,
+                                                                  (float*)out, out_stride, heads, vdim, eps);
+    else
+      delta_readout_norm_kernel<bf16_t><<<ngrid, 256, 0, stream>>>(readout, (const bf16_t*)proj, proj_stride, col_g, norm_weight,
+                                                                   (bf16_t*)out, out_stride, heads, vdim, eps);
+    MI_CHECK_LAUNCH("delta_readout_norm");
+  }
   return MI_OK;
 }

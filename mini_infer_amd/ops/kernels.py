@@ -1590,12 +1590,11 @@ def short_conv(
 
 def delta_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int]:
     """How `gated_delta` lays a request's state out: per head S transposed, [vdim][padded dim].
-    A column is kept by 16, 8 or 4 neighbouring lanes (as many as fit a block of 1,024 threads),
-    each holding 4, 16 or 64 rows: the padded dim is their product (the kernel checks it)."""
-    lanes = 16 if vdim <= 64 else (8 if vdim <= 128 else 4)
-    need = -(-dim // lanes)
-    rows = 4 if need <= 4 else (16 if need <= 16 else 64)
-    return (heads, vdim, lanes * rows)
+    A column is kept by 16 neighbouring lanes, each holding 4, 8 or 16 rows: the padded dim is
+    their product (the kernel checks it)."""
+    need = -(-dim // 16)
+    rows = 4 if need <= 4 else (8 if need <= 8 else 16)
+    return (heads, vdim, 16 * rows)
 
 
 def gated_delta(
@@ -1631,11 +1630,13 @@ def gated_delta(
     if cu_seqlens.numel() != requests + 1:
         raise KernelShapeError("gated_delta: one more boundary than requests")
     out = torch.empty((qkv.shape[0], heads * vdim), dtype=qkv.dtype, device=qkv.device)
+    readout = torch.empty((qkv.shape[0], heads * vdim), dtype=torch.float32, device=qkv.device)  # S^T q before its norm
     library.check(
         library.load().mi_gated_delta(
             _dtype_code(qkv), _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(col_b), int(col_a), int(col_g),
             _ptr(a_log), _ptr(dt_bias), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(slots),
-            _ptr(out), out.stride(0), requests, heads, kv_heads, dim, vdim, shape[2], float(eps), state.shape[0] - 1, _stream(),
+            _ptr(readout), _ptr(out), out.stride(0), qkv.shape[0], requests, heads, kv_heads, dim, vdim, shape[2], float(eps),
+            state.shape[0] - 1, _stream(),
         )
     )
     return out
@@ -1643,16 +1644,20 @@ def gated_delta(
 
 def latent_prepare(
     proj: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, norm_weight: torch.Tensor, slot_mapping: torch.Tensor | None,
-    k_pages: torch.Tensor | None, queries: torch.Tensor, *, heads: int, q_head_width: int, q_rot_at: int, c_col: int,
-    rank: int, rot: int, eps: float,
+    k_pages: torch.Tensor | None, queries: torch.Tensor | None, *, heads: int, q_head_width: int, q_rot_at: int, c_col: int,
+    rank: int, rot: int, eps: float, latent_out: torch.Tensor | None = None,
 ) -> None:
     """What a latent attention layer does between its projections and its attention.  `proj`
     [T, ...] holds the query heads (`q_head_width` columns each from column 0 on, the part to
     rotate `rot` wide from `q_rot_at` inside a head) and from `c_col` on [x_c (rank) | x_r (rot)].
     Writes `[rms_norm(x_c) * norm_weight | rotated x_r]` into the token's slot of `k_pages`
     ([num_pages, 1, page_size, rank + rot]; nothing with `slot_mapping=None`) and each head's
-    rotated query part into the last `rot` columns of its [rank + rot] wide piece of `queries`."""
-    _need_cuda(proj, cos, sin, norm_weight, slot_mapping, k_pages, queries)
+    rotated query part into the last `rot` columns of its [rank + rot] wide piece of `queries`
+    (`queries=None`: not wanted).  `latent_out` [T, rank]: a copy of the normed latents, if wanted."""
+    _need_cuda(proj, cos, sin, norm_weight, slot_mapping, k_pages, queries, latent_out)
+    _need_contiguous("latent_out", latent_out)
+    if latent_out is not None and (latent_out.dtype != proj.dtype or tuple(latent_out.shape) != (proj.shape[0], rank)):
+        raise KernelShapeError(f"latent_prepare: latent_out is {proj.dtype} [{proj.shape[0]}, {rank}], got {latent_out.dtype} {tuple(latent_out.shape)}")
     for name, t in (("cos", cos), ("sin", sin), ("norm_weight", norm_weight), ("slot_mapping", slot_mapping), ("k_pages", k_pages)):
         _need_contiguous(name, t)
     _need_int32("slot_mapping", slot_mapping)
@@ -1660,7 +1665,8 @@ def latent_prepare(
     tokens = proj.shape[0]
     if proj.dim() != 2 or proj.stride(1) != 1 or proj.shape[1] < max(heads * q_head_width, c_col + rank + rot):
         raise KernelShapeError(f"latent_prepare: the projections' rows are too short, got {tuple(proj.shape)}")
-    if queries.dtype != proj.dtype or queries.dim() != 2 or queries.stride(1) != 1 or tuple(queries.shape) != (tokens, heads * (rank + rot)):
+    if queries is not None and (queries.dtype != proj.dtype or queries.dim() != 2 or queries.stride(1) != 1
+                                or tuple(queries.shape) != (tokens, heads * (rank + rot))):
         raise KernelShapeError(f"latent_prepare: queries are {proj.dtype} [{tokens}, {heads * (rank + rot)}], got {queries.dtype} {tuple(queries.shape)}")
     if cos.dtype != torch.float32 or tuple(cos.shape) != (tokens, rot // 2) or sin.shape != cos.shape or sin.dtype != torch.float32:
         raise KernelShapeError(f"latent_prepare: cos/sin must be float32 [{tokens}, {rot // 2}], got {tuple(cos.shape)} {cos.dtype}")
@@ -1675,9 +1681,38 @@ def latent_prepare(
         library.load().mi_latent_prepare(
             _dtype_code(proj), _ptr(proj), proj.stride(0), 0, int(q_head_width), int(q_rot_at), int(c_col), _ptr(cos), _ptr(sin),
             _ptr(norm_weight), _ptr(slot_mapping), _ptr(k_pages) if slot_mapping is not None else None, _ptr(queries),
-            queries.stride(0), tokens, heads, rank, rot, float(eps), _stream(),
+            0 if queries is None else queries.stride(0), _ptr(latent_out), tokens, heads, rank, rot, float(eps), _stream(),
         )
     )
+
+
+def latent_expand(
+    proj: torch.Tensor, k_up: torch.Tensor, v_up: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, *, heads: int,
+    dim: int, rot: int, vdim: int, r_col: int,
+) -> torch.Tensor:
+    """One row [q | k | v] per token with `heads` heads of D = dim + rot columns each, from a latent
+    attention layer's projections (`proj`: query heads [plain (dim) | to rotate (rot)] from column 0
+    on, the shared part to rotate from `r_col` on), the keys' plain parts `k_up` [T, heads*dim] and the
+    values `v_up` [T, heads*vdim] (padded with zeros to D): what the paged attention kernels take."""
+    _need_cuda(proj, k_up, v_up, cos, sin)
+    for name, t in (("proj", proj), ("k_up", k_up), ("v_up", v_up)):
+        if t.dim() != 2 or t.stride(1) != 1 or t.dtype != proj.dtype or t.shape[0] != proj.shape[0]:
+            raise KernelShapeError(f"latent_expand: {name} must be rows of the step in {proj.dtype} with unit inner stride")
+    _need_contiguous("cos", cos)
+    _need_contiguous("sin", sin)
+    tokens, width = proj.shape[0], dim + rot
+    if cos.dtype != torch.float32 or tuple(cos.shape) != (tokens, rot // 2) or sin.shape != cos.shape or sin.dtype != torch.float32:
+        raise KernelShapeError(f"latent_expand: cos/sin must be float32 [{tokens}, {rot // 2}]")
+    if k_up.shape[1] != heads * dim or v_up.shape[1] != heads * vdim or vdim > width or proj.shape[1] < max(heads * width, r_col + rot):
+        raise KernelShapeError("latent_expand: the projections do not hold what the sizes say")
+    qkv = torch.empty((tokens, 3 * heads * width), dtype=proj.dtype, device=proj.device)
+    library.check(
+        library.load().mi_latent_expand(
+            _dtype_code(proj), _ptr(proj), proj.stride(0), width, dim, int(r_col), _ptr(k_up), k_up.stride(0), _ptr(v_up),
+            v_up.stride(0), _ptr(cos), _ptr(sin), _ptr(qkv), qkv.stride(0), tokens, heads, dim, rot, vdim, _stream(),
+        )
+    )
+    return qkv
 
 
 def linear_per_head(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:

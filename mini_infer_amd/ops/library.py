@@ -14,7 +14,7 @@ from pathlib import Path
 from mini_infer_amd.exceptions import ExtensionMissingError, KernelShapeError
 from mini_infer_amd.ops import build as _build
 
-ABI_VERSION = 26
+ABI_VERSION = 28
 
 _lib: ctypes.CDLL | None = None
 _lib_path: Path | None = None
@@ -85,13 +85,17 @@ _SIGNATURES: dict[str, list] = {
     "mi_clamped_glu": [c_int, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_float, _P],
     "mi_short_conv": [c_int, _P, c_int64, _P, _P, c_int64, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P],
     "mi_gated_delta": [
-        c_int, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int64, _P, _P, _P, c_int64,
-        c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
+        c_int, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int64,
+        c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P,
     ],
     "mi_gated_delta_rows": [c_int, c_int],
     "mi_latent_prepare": [
-        c_int, _P, c_int64, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
+        c_int, _P, c_int64, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int64, _P, c_int, c_int, c_int, c_int,
         c_float, _P,
+    ],
+    "mi_latent_expand": [
+        c_int, _P, c_int64, c_int, c_int, c_int, _P, c_int64, _P, c_int64, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
+        c_int, _P,
     ],
 }
 

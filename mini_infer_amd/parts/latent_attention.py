@@ -9,11 +9,17 @@ beside it one rotated key part `r` of `rot_dim` numbers is shared by all heads:
     out = W_o concat_a( sum_j softmax_j(score_a(i, .)) W_uv,a c(j) )
 
 Only `[c | r]` is cached: one key head of `kv_rank + rot_dim` numbers a token, whatever the
-number of heads.  The key map is folded into the query, `q'_a = W_uk,a^T q_a,plain`, so a
-head's score is `[q'_a | q_a,rot] . [c | r]`, and the value map is applied after the
-attention, `W_uv,a (sum_j p_j c(j))`: the attention itself is the paged kernel with a single
-key/value head whose value row is the front part of its key row.  Prompts and single tokens
-take the same path, so a position's result does not depend on how its prompt was cut.
+number of heads.  Over the cache the key map is folded into the query, `q'_a = W_uk,a^T
+q_a,plain`, so a head's score is `[q'_a | q_a,rot] . [c | r]`, and the value map is applied
+after the attention, `W_uv,a (sum_j p_j c(j))`: the attention itself is the paged kernel with
+a single key/value head whose value row is the front part of its key row.
+
+A step in which every request begins (prompts that come whole, or first portions) has all its
+keys at hand, and there the folded form is the dearer one: every head would score against
+kv_rank + rot_dim numbers a key instead of head_dim + rot_dim.  Such a step writes keys and
+values out per head into pages of its own and runs the matrix-core attention kernel over them
+like any other layer (bfloat16, head sizes it takes); the cache gets the same `[c | r]` rows
+either way.  The two forms differ by rounding only.
 """
 
 from __future__ import annotations
@@ -73,6 +79,7 @@ class LatentAttention(Mixer):
         self.latent_norm: torch.Tensor | None = None
         self.fold_k: torch.Tensor | None = None  # [heads, kv_rank, head_dim]: W_uk,a transposed
         self.map_v: torch.Tensor | None = None  # [heads, v_head_dim, kv_rank]
+        self._out_padded: torch.Tensor | None = None  # W_o with zero columns where expanded value heads are padded
 
     def param_specs(self, prefix: str) -> dict[str, ParamSpec]:
         return {
@@ -90,11 +97,76 @@ class LatentAttention(Mixer):
         assert self.up_k.weight is not None and self.up_v.weight is not None
         self.fold_k = self.up_k.weight.view(self.num_heads, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
         self.map_v = self.up_v.weight.view(self.num_heads, self.v_head_dim, self.kv_rank)
-        self.up_k.weight = None  # (kept transposed only)
+        self._out_padded = None
 
     def cache_needs(self, page_size: int) -> CacheNeeds:
         # one key head, rows [c | r]; the values are the rows' front part: no value pages
         return CacheNeeds(pages=PagedKVNeeds(1, self.kv_rank + self.rot_dim, None, v_head_dim=0))
+
+    EXPAND_MIN_TOKENS = 64  # steps of fewer tokens take the folded form whatever they hold
+
+    def _expands(self, ctx: StepContext) -> bool:
+        """Whether this step writes keys and values out per head: every request begins in it (known
+        on the host), and the matrix-core attention kernel takes the sizes."""
+        width = self.head_dim + self.rot_dim
+        if self.dtype != torch.bfloat16 or ctx.host_cu_seqlens_q is None or ctx.host_seq_lens is None:
+            return False
+        if ctx.num_tokens < self.EXPAND_MIN_TOKENS or self.v_head_dim > width:
+            return False
+        if not ops.mfma_attention_supported(self.dtype, width, ctx.page_size):
+            return False
+        cu = ctx.host_cu_seqlens_q
+        return all(ctx.host_seq_lens[b] == cu[b + 1] - cu[b] for b in range(len(ctx.host_seq_lens)))
+
+    def _own_pages(self, ctx: StepContext) -> tuple[torch.Tensor, torch.Tensor, int]:
+        """Write slots, block table and page count of pages that hold this step's tokens alone, each
+        request from a page of its own on (made once a step, on the host, for all layers that expand)."""
+        key = ("latent_attention_own_pages", ctx.page_size)
+        if key not in ctx.shared:
+            import numpy as np
+
+            cu, page = np.asarray(ctx.host_cu_seqlens_q, dtype=np.int64), ctx.page_size
+            lengths = cu[1:] - cu[:-1]
+            pages = -(-lengths // page)
+            first = np.concatenate([[0], np.cumsum(pages)])
+            request_of = np.repeat(np.arange(len(lengths)), lengths)
+            slots = first[request_of] * page + (np.arange(cu[-1]) - cu[request_of])
+            table = np.zeros((len(lengths), max(1, int(pages.max()))), dtype=np.int32)
+            for b, count in enumerate(pages):
+                table[b, :count] = first[b] + np.arange(count)
+            both = torch.from_numpy(np.concatenate([slots.astype(np.int32), table.reshape(-1)])).to(self.device)
+            ctx.shared[key] = (both[: slots.size], both[slots.size:].view(table.shape), int(first[-1]))
+        return ctx.shared[key]
+
+    def _forward_expanded(self, proj: torch.Tensor, ctx: StepContext, cache: LayerCache, writes_cache: bool) -> torch.Tensor:
+        heads, rank, rot, dim, vdim = self.num_heads, self.kv_rank, self.rot_dim, self.head_dim, self.v_head_dim
+        width, tokens = dim + rot, proj.shape[0]
+        rotary = self.position.rotary(ctx)
+        latent = torch.empty((tokens, rank), dtype=proj.dtype, device=proj.device)
+        ops.latent_prepare(
+            proj, rotary.cos, rotary.sin, self.latent_norm, ctx.slot_mapping[cache.group] if writes_cache else None,
+            cache.k_pages, None, heads=heads, q_head_width=self.q_head_width, q_rot_at=dim, c_col=heads * self.q_head_width,
+            rank=rank, rot=rot, eps=self.norm_eps, latent_out=latent,
+        )
+        qkv = ops.latent_expand(proj, self.up_k.forward(latent), self.up_v.forward(latent), rotary.cos, rotary.sin, heads=heads,
+                                dim=dim, rot=rot, vdim=vdim, r_col=heads * self.q_head_width + rank)
+        slots, table, pages = self._own_pages(ctx)
+        # (zeroed: the kernel multiplies what lies past a request's last key by a weight of zero)
+        k_own = torch.zeros((pages, heads, ctx.page_size, width), dtype=proj.dtype, device=proj.device)
+        v_own = torch.zeros((pages, heads, width, ctx.page_size), dtype=proj.dtype, device=proj.device)
+        nothing = torch.empty((tokens, 0), dtype=torch.float32, device=proj.device)
+        ops.rope_kv_write(qkv, nothing, nothing, slots, k_own, v_own, q_heads=heads, kv_heads=heads, head_dim=width,
+                          rotary_dim=0, v_transposed=True)
+        mixed = ops.paged_attention(
+            qkv, k_own, v_own, table, ctx.token_request, ctx.positions, ctx.cu_seqlens_q, ctx.host_cu_seqlens_q, q_heads=heads,
+            kv_heads=heads, head_dim=width, scale=self.scale, window=None, max_seq_len=ctx.max_q_len, v_transposed=True,
+        )
+        if self._out_padded is None:  # W_o with zero columns under the padding of every value head
+            assert self.out.weight is not None
+            padded = torch.zeros((self.hidden_size, heads, width), dtype=self.out.weight.dtype, device=self.out.weight.device)
+            padded[:, :, :vdim] = self.out.weight.view(self.hidden_size, heads, vdim)
+            self._out_padded = padded.view(self.hidden_size, heads * width)
+        return ops.linear(mixed, self._out_padded)
 
     def forward(self, x, ctx: StepContext, cache: LayerCache, writes_cache: bool = True):
         assert cache.group is not None and cache.k_pages is not None
@@ -104,6 +176,8 @@ class LatentAttention(Mixer):
             x = x.finish()
         heads, rank, rot, width = self.num_heads, self.kv_rank, self.rot_dim, self.kv_rank + self.rot_dim
         proj = self.q_down.forward(x)
+        if self._expands(ctx):
+            return self._forward_expanded(proj, ctx, cache, writes_cache)
         tokens = proj.shape[0]
         rotary = self.position.rotary(ctx)
         queries = torch.empty((tokens, heads * width), dtype=proj.dtype, device=proj.device)

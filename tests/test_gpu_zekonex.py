@@ -319,6 +319,27 @@ def test_logits_do_not_depend_on_the_schedule(folders, name, dtype, family):
     assert runner.num_free_blocks() == pages
 
 
+def test_prompts_that_come_whole_write_keys_and_values_out_per_head(folders, monkeypatch):
+    """bfloat16, a latent attention layer whose head sizes the matrix-core kernel takes: a step in
+    which every request begins takes the expanded form (two prompts side by side, neither filling
+    its last page), any other step the folded one; both agree with the plain model."""
+    from mini_infer_amd.engine import StepEntry
+    from mini_infer_amd.parts.latent_attention import LatentAttention
+
+    cfg, block, weights, folder = folders["C"]
+    calls = []
+    original = LatentAttention._forward_expanded
+    monkeypatch.setattr(LatentAttention, "_forward_expanded", lambda self, *a, **k: (calls.append(1), original(self, *a, **k))[1])
+    runner = runner_for(folder, "bfloat16", block, pages=24, seats=2)
+    first, second = tz.random_tokens(cfg, 101, seed=5), tz.random_tokens(cfg, 70, seed=6)
+    both = runner.step([StepEntry("p", first[:90], list(range(90))), StepEntry("q", second, list(range(70)))]).cpu().numpy()
+    assert len(calls) == 1  # (one latent attention layer in this configuration)
+    rest = runner.step([StepEntry("p", first[90:], list(range(11)))]).cpu().numpy()
+    assert len(calls) == 1  # a later portion reads the cache: folded
+    ru.assert_close(np.concatenate([both[:90], rest]), oracle("C", cfg, weights, first), "bfloat16", "whole then a portion")
+    ru.assert_close(both[90:], oracle("C", cfg, weights, second), "bfloat16", "beside it")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_slot_and_pages_used_again_start_clean(folders, dtype):
     """One seat, pages for one request: the second request gets the first one's slot (recurrent
