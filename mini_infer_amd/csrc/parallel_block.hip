@@ -35,9 +35,65 @@ __device__ __forceinline__ double block_sum_wide(double v, double* scratch) {
   return total;
 }
 
+typedef bf16_t bf16x4_t __attribute__((ext_vector_type(4)));
+
+// VEC consecutive elements at once (VEC = 4: 16-byte float32 and 8-byte bfloat16 accesses)
+template <int VEC>
+__device__ __forceinline__ void load_some(const float* p, float v[VEC]) {
+  if constexpr (VEC == 4) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+  } else {
+    v[0] = p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void load_some(const bf16_t* p, float v[VEC]) {
+  if constexpr (VEC == 4) {
+    const bf16x4_t x = *reinterpret_cast<const bf16x4_t*>(p);
+    v[0] = (float)x[0], v[1] = (float)x[1], v[2] = (float)x[2], v[3] = (float)x[3];
+  } else {
+    v[0] = (float)p[0];
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void store_some(float* p, const float v[VEC]) {
+  if constexpr (VEC == 4) *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  else p[0] = v[0];
+}
+template <int VEC>
+__device__ __forceinline__ void store_some(bf16_t* p, const float v[VEC]) {
+  if constexpr (VEC == 4) {
+    bf16x4_t x;
+    x[0] = (bf16_t)v[0], x[1] = (bf16_t)v[1], x[2] = (bf16_t)v[2], x[3] = (bf16_t)v[3];
+    *reinterpret_cast<bf16x4_t*>(p) = x;
+  } else {
+    p[0] = (bf16_t)v[0];
+  }
+}
+
+// The new values of VEC columns of a row: x + scale * (a + b + bias) + shift.
+template <typename T, int VEC>
+__device__ __forceinline__ void updated(const T* ar, const T* br, const float* bias, const float* shift, float scale,
+                                        const float* x, int c, float value[VEC]) {
+  float xv[VEC], av[VEC], bv[VEC], cv[VEC], sv[VEC];
+  load_some<VEC>(x + c, xv);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) av[e] = bv[e] = cv[e] = sv[e] = 0.f;
+  if (ar) load_some<VEC>(ar + c, av);
+  if (br) load_some<VEC>(br + c, bv);
+  if (bias) load_some<VEC>(bias + c, cv);
+  if (shift) load_some<VEC>(shift + c, sv);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    if constexpr (sizeof(T) == 4) value[e] = (float)((double)xv[e] + (double)scale * (((double)av[e] + (double)bv[e]) + (double)cv[e]) + (double)sv[e]);
+    else value[e] = xv[e] + scale * ((av[e] + bv[e]) + cv[e]) + sv[e];
+  }
+}
+
 // One block a row.  `rows` (optional) lists the rows to norm; with it the stream is left as
 // it was (the rows' new values are used for the norm only), as the final norm wants it.
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(1024) void stream_update_norm_kernel(
     const T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
     const float* __restrict__ bias, const float* __restrict__ shift, float scale, float* __restrict__ stream,
@@ -50,34 +106,25 @@ __global__ __launch_bounds__(1024) void stream_update_norm_kernel(
   float* x = stream + (int64_t)t * hidden;
   const T* ar = a ? a + (int64_t)t * a_stride : nullptr;
   const T* br = b ? b + (int64_t)t * b_stride : nullptr;
-  // a thread keeps its columns' new values (up to 8 of them; wider rows are read again)
-  constexpr int KEEP = 8;
-  float kept[KEEP];
+  // a thread keeps the new values of its first columns (wider rows are made again below)
+  constexpr int KEEP = 4;
+  float kept[KEEP][VEC];
   float squares = 0.f;
   double squares_wide = 0.0;
   int n = 0;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x, ++n) {
-    float value;
-    if constexpr (WIDE) {
-      double sum = 0.0;
-      if (ar) sum += (double)ar[c];
-      if (br) sum += (double)br[c];
-      if (bias) sum += (double)bias[c];
-      double v = (double)x[c] + (double)scale * sum;
-      if (shift) v += (double)shift[c];
-      value = (float)v;
-      squares_wide += (double)value * (double)value;
-    } else {
-      float sum = 0.f;
-      if (ar) sum += to_f32(ar[c]);
-      if (br) sum += to_f32(br[c]);
-      if (bias) sum += bias[c];
-      value = x[c] + scale * sum;
-      if (shift) value += shift[c];
-      squares += value * value;
+  for (int c = threadIdx.x * VEC; c < hidden; c += blockDim.x * VEC, ++n) {
+    float value[VEC];
+    updated<T, VEC>(ar, br, bias, shift, scale, x, c, value);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if constexpr (WIDE) squares_wide += (double)value[e] * (double)value[e];
+      else squares += value[e] * value[e];
     }
-    if (!rows) x[c] = value;
-    if (n < KEEP) kept[n] = value;
+    if (!rows) store_some<VEC>(x + c, value);
+    if (n < KEEP) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) kept[n][e] = value[e];
+    }
   }
   if (!weight) return;
   float inv;
@@ -90,56 +137,56 @@ __global__ __launch_bounds__(1024) void stream_update_norm_kernel(
   }
   T* o = out + (int64_t)r * hidden;
   n = 0;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x, ++n) {
-    float value;
+  for (int c = threadIdx.x * VEC; c < hidden; c += blockDim.x * VEC, ++n) {
+    float value[VEC], w[VEC];
     if (n < KEEP) {
-      value = kept[n];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) value[e] = kept[n][e];
     } else if (!rows) {
-      value = x[c];
-    } else {  // recompute: the stream was not written
-      if constexpr (WIDE) {
-        double sum = 0.0;
-        if (ar) sum += (double)ar[c];
-        if (br) sum += (double)br[c];
-        if (bias) sum += (double)bias[c];
-        double v = (double)x[c] + (double)scale * sum;
-        if (shift) v += (double)shift[c];
-        value = (float)v;
-      } else {
-        float sum = 0.f;
-        if (ar) sum += to_f32(ar[c]);
-        if (br) sum += to_f32(br[c]);
-        if (bias) sum += bias[c];
-        value = x[c] + scale * sum;
-        if (shift) value += shift[c];
-      }
+      load_some<VEC>(x + c, value);
+    } else {  // made again: the stream was not written
+      updated<T, VEC>(ar, br, bias, shift, scale, x, c, value);
     }
-    if constexpr (WIDE) o[c] = (float)((double)value * inv_wide * (double)weight[c]);
-    else o[c] = from_f32<T>(value * inv * to_f32(weight[c]));
+    load_some<VEC>(weight + c, w);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      if constexpr (WIDE) value[e] = (float)((double)value[e] * inv_wide * (double)w[e]);
+      else value[e] = value[e] * inv * w[e];
+    }
+    store_some<VEC>(o + c, value);
   }
 }
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ gate_up, int64_t in_stride,
                                                           const float* __restrict__ bias, T* __restrict__ out,
                                                           int64_t out_stride, int inter, float limit, float slope) {
   const int t = blockIdx.y;
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (c >= inter) return;
   const T* row = gate_up + (int64_t)t * in_stride;
-  if constexpr (sizeof(T) == 4) {
-    double g = (double)row[c] + (bias ? (double)bias[c] : 0.0);
-    double u = (double)row[inter + c] + (bias ? (double)bias[inter + c] : 0.0);
-    g = fmin(g, (double)limit);
-    u = fmin(fmax(u, -(double)limit), (double)limit);
-    out[(int64_t)t * out_stride + c] = (float)(g / (1.0 + exp(-(double)slope * g)) * (u + 1.0));
-  } else {
-    float g = to_f32(row[c]) + (bias ? bias[c] : 0.f);
-    float u = to_f32(row[inter + c]) + (bias ? bias[inter + c] : 0.f);
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    out[(int64_t)t * out_stride + c] = from_f32<T>(g * mi_logistic(slope * g) * (u + 1.f));
+  float g[VEC], u[VEC], bg[VEC], bu[VEC], y[VEC];
+  load_some<VEC>(row + c, g);
+  load_some<VEC>(row + inter + c, u);
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) bg[e] = bu[e] = 0.f;
+  if (bias) {
+    load_some<VEC>(bias + c, bg);
+    load_some<VEC>(bias + inter + c, bu);
   }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    if constexpr (sizeof(T) == 4) {
+      double gd = fmin((double)g[e] + (double)bg[e], (double)limit);
+      double ud = fmin(fmax((double)u[e] + (double)bu[e], -(double)limit), (double)limit);
+      y[e] = (float)(gd / (1.0 + exp(-(double)slope * gd)) * (ud + 1.0));
+    } else {
+      const float gf = fminf(g[e] + bg[e], limit);
+      const float uf = fminf(fmaxf(u[e] + bu[e], -limit), limit);
+      y[e] = gf * mi_logistic(slope * gf) * (uf + 1.f);
+    }
+  }
+  store_some<VEC>(out + (int64_t)t * out_stride + c, y);
 }
 
 }  // namespace
@@ -160,14 +207,17 @@ extern "C" int mi_stream_update_norm(int dtype, const void* a, int64_t a_stride,
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "stream_update_norm: unknown dtype %d", dtype);
   if (num_out_rows == 0) return MI_OK;
   const int threads = (num_out_rows <= 64 && hidden >= 2048) ? 1024 : 256;
-  if (dtype == MI_F32)
-    stream_update_norm_kernel<float><<<num_out_rows, threads, 0, stream_handle>>>(
-        (const float*)a, a_stride, (const float*)b, b_stride, bias, shift, scale, stream, (const float*)weight,
-        (float*)out, rows, hidden, eps);
-  else
-    stream_update_norm_kernel<bf16_t><<<num_out_rows, threads, 0, stream_handle>>>(
-        (const bf16_t*)a, a_stride, (const bf16_t*)b, b_stride, bias, shift, scale, stream, (const bf16_t*)weight,
-        (bf16_t*)out, rows, hidden, eps);
+  // four columns a thread where every row begins on a 16-byte boundary
+  const size_t elem = dtype == MI_F32 ? 4 : 2;
+  const bool vec = hidden % 4 == 0 && ((uintptr_t)a | (uintptr_t)b | (uintptr_t)weight | (uintptr_t)out | (uintptr_t)(a_stride * elem) |
+                                       (uintptr_t)(b_stride * elem)) % 16 == 0 &&
+                   ((uintptr_t)bias | (uintptr_t)shift | (uintptr_t)stream) % 16 == 0;
+#define MI_UPDATE_LAUNCH(T, VEC)                                                                                      \
+  stream_update_norm_kernel<T, VEC><<<num_out_rows, threads, 0, stream_handle>>>(                                     \
+      (const T*)a, a_stride, (const T*)b, b_stride, bias, shift, scale, stream, (const T*)weight, (T*)out, rows, hidden, eps)
+  if (dtype == MI_F32) { if (vec) MI_UPDATE_LAUNCH(float, 4); else MI_UPDATE_LAUNCH(float, 1); }
+  else { if (vec) MI_UPDATE_LAUNCH(bf16_t, 4); else MI_UPDATE_LAUNCH(bf16_t, 1); }
+#undef MI_UPDATE_LAUNCH
   MI_CHECK_LAUNCH("stream_update_norm");
   return MI_OK;
 }
@@ -182,18 +232,19 @@ extern "C" int mi_clamped_glu(int dtype, const void* gate_up, int64_t in_stride,
   MI_REQUIRE(num_tokens <= 65535 * 64, "clamped_glu: too many tokens");
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "clamped_glu: unknown dtype %d", dtype);
   if (num_tokens == 0) return MI_OK;
+  const size_t elem = dtype == MI_F32 ? 4 : 2;
+  const bool vec = inter % 4 == 0 && ((uintptr_t)gate_up | (uintptr_t)out | (uintptr_t)(in_stride * elem) | (uintptr_t)(out_stride * elem) |
+                                      (uintptr_t)(inter * elem)) % 16 == 0 && (uintptr_t)bias % 16 == 0;
   // (rows along y in slices of at most 65535)
   for (int first = 0; first < num_tokens; first += 65535) {
     const int count = min(65535, num_tokens - first);
-    dim3 grid(ceil_div(inter, 256), count);
-    if (dtype == MI_F32)
-      clamped_glu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up + (int64_t)first * in_stride, in_stride, bias,
-                                                          (float*)out + (int64_t)first * out_stride, out_stride, inter,
-                                                          limit, slope);
-    else
-      clamped_glu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up + (int64_t)first * in_stride, in_stride,
-                                                           bias, (bf16_t*)out + (int64_t)first * out_stride, out_stride,
-                                                           inter, limit, slope);
+    dim3 grid(ceil_div(inter, 256 * (vec ? 4 : 1)), count);
+#define MI_GLU_LAUNCH(T, VEC)                                                                                          \
+  clamped_glu_kernel<T, VEC><<<grid, 256, 0, stream>>>((const T*)gate_up + (int64_t)first * in_stride, in_stride, bias, \
+                                                       (T*)out + (int64_t)first * out_stride, out_stride, inter, limit, slope)
+    if (dtype == MI_F32) { if (vec) MI_GLU_LAUNCH(float, 4); else MI_GLU_LAUNCH(float, 1); }
+    else { if (vec) MI_GLU_LAUNCH(bf16_t, 4); else MI_GLU_LAUNCH(bf16_t, 1); }
+#undef MI_GLU_LAUNCH
   }
   MI_CHECK_LAUNCH("clamped_glu");
   return MI_OK;

@@ -111,8 +111,10 @@ class LatentAttention(Mixer):
         width = self.head_dim + self.rot_dim
         if self.dtype != torch.bfloat16 or ctx.host_cu_seqlens_q is None or ctx.host_seq_lens is None:
             return False
-        if ctx.num_tokens < self.EXPAND_MIN_TOKENS or self.v_head_dim > width:
-            return False
+        if ctx.num_tokens < self.EXPAND_MIN_TOKENS or ctx.max_q_len < 2 or self.v_head_dim > width:
+            return False  # (a step of single tokens that is being recorded says nothing true about lengths)
+        if torch.cuda.is_current_stream_capturing():
+            return False  # (this form makes its index on the host)
         if not ops.mfma_attention_supported(self.dtype, width, ctx.page_size):
             return False
         cu = ctx.host_cu_seqlens_q
