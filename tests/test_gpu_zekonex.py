@@ -287,7 +287,8 @@ def test_each_mixer_alone_whole_and_token_by_token(tmp_path, dtype, mixer):
 # whole models under every kind of schedule
 # ---------------------------------------------------------------------------------------------
 
-LENGTHS = {"A": (70, 41, 9, 33, 58, 1), "B": (45, 64, 17, 2, 39), "C": (130, 40, 77, 5), "D": (50, 21, 36, 3, 44)}
+LENGTHS = {"A": (70, 41, 9, 33, 58, 1), "B": (45, 64, 17, 2, 39), "C": (130, 40, 77, 5), "D": (50, 21, 36, 3, 44),
+           "E": (90, 35, 66, 3)}
 
 
 def requests_of(name, cfg):

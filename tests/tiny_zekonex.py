@@ -82,7 +82,22 @@ TINY_D = config(97, 48, [delta(2, 2, 8, 8, 4, ff=64, limit=1.0), delta(3, 1, 20,
                 loop=(0, 2, 2))
 TINY_D_BLOCK = 4
 
-CONFIGS = {"A": (TINY_A, TINY_A_BLOCK), "B": (TINY_B, TINY_B_BLOCK), "C": (TINY_C, TINY_C_BLOCK), "D": (TINY_D, TINY_D_BLOCK)}
+# the largest heads the kernels take and the corners of their fast paths: a latent layer whose value
+# heads are wider than its expanded key heads (prompts then take the folded form in bfloat16 too) and one
+# with the smallest head size the matrix cores take; attention heads of 128 with a sink on the matrix
+# cores, and value heads half as wide as the query heads (plain kernel); a delta rule of 256 x 256 with two
+# taps; the loop runs to the last layer
+TINY_E = config(200, 128, [
+    attention(2, 2, 128, 128, 0.12, rot=(10000.0, 128), ff=192, limit=2.5),
+    latent(2, 48, 16, 96, 40, 0.3, 300.0, ff=64, limit=1.0),
+    delta(2, 1, 256, 256, 2),
+    latent(2, 24, 8, 16, 64, 0.4, 20000.0),
+    attention(4, 1, 64, 32, 0.25, rot=(50.0, 2), ff=96, limit=0.9),
+], scale=4.0, eps=1e-6, mult=0.4, loop=(1, 5, 3))
+TINY_E_BLOCK = 16
+
+CONFIGS = {"A": (TINY_A, TINY_A_BLOCK), "B": (TINY_B, TINY_B_BLOCK), "C": (TINY_C, TINY_C_BLOCK), "D": (TINY_D, TINY_D_BLOCK),
+           "E": (TINY_E, TINY_E_BLOCK)}
 
 
 def bf16_round(values: np.ndarray) -> np.ndarray:
