@@ -68,7 +68,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 //              The norm's launch between two products is saved.
 // In every case the sums are rounded to bfloat16 before the activation or rotation,
 // exactly as when the product and the second step run as two kernels.
-enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5, EPI_GRU = 6 };
+enum { EPI_STORE = 0, EPI_GATED = 1, EPI_ROPE = 2, EPI_ADDNORM = 3, EPI_STORE_F32 = 4, EPI_GELU_TABLE = 5, EPI_GRU = 6,
+       EPI_GATED_CLAMPED = 7 };
 // Where the activations come from: a matrix in memory, or (PRO_ATTN, few rows) the
 // uncombined key ranges of attn_mfma: each wave first combines its own columns of the
 // attention output (what attn_reduce would have written) into LDS, so the combining launch
@@ -112,6 +113,10 @@ struct FoldArgs {  // what the folded neighbours of a product need
   int64_t ld_table;
   const int* table_ids;
   int table_col;
+  // EPI_GATED_CLAMPED: float32 [2n] biases of gate and up,
+  // out = g * logistic(slope * g) * (u + 1), g = min(gate + bias, limit), u = clamp(up + bias, -limit, limit)
+  const float* glu_bias;
+  float glu_limit, glu_slope;
   // PRO_SCALED: the pieces of the rows' sums of squares [pieces][m], the norm's eps and width
   const float* sumsq_in;
   int sumsq_pieces;
@@ -123,7 +128,7 @@ template <int NT, int U, int EPI, int PRO = PRO_NONE, bool LINES = false, int RT
 __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
     const bf16_t* __restrict__ a, int64_t lda, const bf16_t* __restrict__ w, int64_t ldw,
     bf16_t* __restrict__ c, int64_t ldc, int m, int n, int k, int features_per_block, const FoldArgs fold) {
-  constexpr bool GATED = EPI == EPI_GATED;
+  constexpr bool GATED = EPI == EPI_GATED || EPI == EPI_GATED_CLAMPED;
   constexpr bool ROPE = EPI == EPI_ROPE;
   constexpr bool ADDNORM = EPI == EPI_ADDNORM;
   constexpr bool SCALED = PRO == PRO_SCALED;
@@ -451,10 +456,21 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_bf16_kernel(
       }
     }
     if (GATED) {
+      if constexpr (EPI == EPI_GATED_CLAMPED) {  // (the arithmetic of clamped_glu on the rounded products, bit for bit)
+        const int feature = n0 + nt * 16 + fq * 4;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float g = (float)(bf16_t)sum[r];
-        sum[r] = g / (1.f + expf(-g)) * (float)(bf16_t)up[r];
+        for (int r = 0; r < 4; ++r) {
+          const int at = min(feature + r, n - 1);
+          const float g = fminf((float)(bf16_t)sum[r] + fold.glu_bias[at], fold.glu_limit);
+          const float u = fminf(fmaxf((float)(bf16_t)up[r] + fold.glu_bias[n + at], -fold.glu_limit), fold.glu_limit);
+          sum[r] = g * mi_logistic(fold.glu_slope * g) * (u + 1.f);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = (float)(bf16_t)sum[r];
+          sum[r] = g / (1.f + expf(-g)) * (float)(bf16_t)up[r];
+        }
       }
     }
     if constexpr (ADDNORM) {
@@ -853,9 +869,33 @@ extern "C" int mi_gemm_skinny_swiglu_scaled_bf16(const void* a, int64_t lda, con
   return MI_OK;
 }
 
+template <int EPI>
+static int skinny_gated(const void* a, int64_t lda, const void* w, int64_t ldw, void* out, int64_t ldo, int m, int n,
+                        int k, const FoldArgs& nothing_folded, hipStream_t stream);
+
 // out[m, n] = silu(a . gate^T) * (a . up^T) with w = [gate; up] stacked, [2n, k].
 extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, void* out,
                                           int64_t ldo, int m, int n, int k, hipStream_t stream) {
+  const FoldArgs nothing_folded = {};
+  return skinny_gated<EPI_GATED>(a, lda, w, ldw, out, ldo, m, n, k, nothing_folded, stream);
+}
+
+// out[m, n] = g * logistic(slope * g) * (u + 1), g = min(a . gate^T + bias[:n], limit), u = clamp(a . up^T +
+// bias[n:], -limit, limit), with w = [gate; up] stacked, [2n, k], and bias float32 [2n].
+extern "C" int mi_gemm_skinny_clamped_glu_bf16(const void* a, int64_t lda, const void* w, int64_t ldw, const float* bias,
+                                               float limit, float slope, void* out, int64_t ldo, int m, int n, int k,
+                                               hipStream_t stream) {
+  MI_REQUIRE(bias != nullptr && limit > 0.f, "gemm_skinny_clamped_glu_bf16: needs the biases and a positive limit");
+  FoldArgs fold = {};
+  fold.glu_bias = bias;
+  fold.glu_limit = limit;
+  fold.glu_slope = slope;
+  return skinny_gated<EPI_GATED_CLAMPED>(a, lda, w, ldw, out, ldo, m, n, k, fold, stream);
+}
+
+template <int EPI>
+static int skinny_gated(const void* a, int64_t lda, const void* w, int64_t ldw, void* out, int64_t ldo, int m, int n,
+                        int k, const FoldArgs& nothing_folded, hipStream_t stream) {
   MI_REQUIRE(mi_gemm_skinny_wide_bf16_supported(m, n, k, lda, ldw),
              "gemm_skinny_swiglu_bf16: takes 1 <= m <= 32, k a multiple of 32, rows aligned to 16 bytes; "
              "got m=%d n=%d k=%d lda=%lld ldw=%lld", m, n, k, (long long)lda, (long long)ldw);
@@ -863,7 +903,6 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const bf16_t* ap = (const bf16_t*)a;
   const bf16_t* wp = (const bf16_t*)w;
   bf16_t* cp = (bf16_t*)out;
-  const FoldArgs nothing_folded = {};
   const int cus = compute_units();
   MI_REQUIRE(cus > 0, "gemm_skinny_swiglu_bf16: cannot read the device's compute unit count");
   const int fpb = features_per_block_for(n, cus, 2);  // two output tiles = four weight tiles
@@ -871,7 +910,7 @@ extern "C" int mi_gemm_skinny_swiglu_bf16(const void* a, int64_t lda, const void
   const int threads = 64 * SK_WAVES;
   const bool lines = whole_lines(w, ldw, 2 * (int64_t)n, k);
 #define SK_GATED(NT_, U_, LINES_, RT_) \
-  gemm_skinny_bf16_kernel<NT_, U_, EPI_GATED, PRO_NONE, LINES_, RT_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded)
+  gemm_skinny_bf16_kernel<NT_, U_, EPI, PRO_NONE, LINES_, RT_><<<blocks, threads, 0, stream>>>(ap, lda, wp, ldw, cp, ldo, m, n, k, fpb, nothing_folded)
   if (m <= 16) {
     if (fpb <= 16) {
       if (lines) SK_GATED(1, 4, true, 1); else SK_GATED(1, 4, false, 1);

@@ -1551,6 +1551,38 @@ def clamped_glu(gate_up: torch.Tensor, bias: torch.Tensor | None, limit: float, 
     return out
 
 
+def linear_clamped_glu(x: torch.Tensor, gate_up_weight: torch.Tensor, bias: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
+    """`clamped_glu(x @ [gate; up].T, bias, limit, slope)`.  bfloat16 with at most 32 rows runs as ONE
+    kernel (the weight-streaming product with biases, clamps and activation in its last step);
+    otherwise the product and `clamped_glu` run in turn.  Both round the two products to the element
+    type first and then do the same float32 arithmetic, so the results agree bit for bit."""
+    rows, width = gate_up_weight.shape
+    if rows % 2 or bias.numel() != rows:
+        raise KernelShapeError(f"linear_clamped_glu: stacked weight of {rows} rows, bias of {bias.numel()}")
+    if (
+        x.dtype == torch.bfloat16
+        and gate_up_weight.dtype == torch.bfloat16
+        and x.dim() == 2
+        and x.shape[1] == width
+        and x.stride(1) == 1
+        and gate_up_weight.stride(1) == 1
+        and skinny_gemm_takes(x.shape[0], width, x.stride(0), gate_up_weight.stride(0), SKINNY_WIDE_MAX_ROWS)
+    ):
+        _need_cuda(x, gate_up_weight, bias)
+        _need_contiguous("bias", bias)
+        _need_f32("bias", bias)
+        m, n = x.shape[0], rows // 2
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        library.check(
+            library.load().mi_gemm_skinny_clamped_glu_bf16(
+                _ptr(x), x.stride(0), _ptr(gate_up_weight), gate_up_weight.stride(0), _ptr(bias), float(limit), float(slope),
+                _ptr(out), out.stride(0), m, n, width, _stream(),
+            )
+        )
+        return out
+    return clamped_glu(linear(x, gate_up_weight), bias, limit, slope)
+
+
 def short_conv(
     x: torch.Tensor, channels: int, taps_weight: torch.Tensor, tail: torch.Tensor, cu_seqlens: torch.Tensor,
     slots: torch.Tensor, token_request: torch.Tensor,

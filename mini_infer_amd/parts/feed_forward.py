@@ -230,7 +230,9 @@ class ClampedGatedFeedForward(FeedForward):
         assert self.gate_up_bias is not None, "feed-forward used before its weights were loaded"
         if isinstance(x, ops.ScaledRows):
             x = x.finish()
-        act = ops.clamped_glu(self.gate_up.forward(x), self.gate_up_bias, self.limit, self.slope)
+        assert self.gate_up.weight is not None
+        # (few rows: the product, the biases, the clamps and the activation are one kernel)
+        act = ops.linear_clamped_glu(x, self.gate_up.weight, self.gate_up_bias, self.limit, self.slope)
         return self.down.forward(act)
 
 

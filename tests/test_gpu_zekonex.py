@@ -122,6 +122,24 @@ def test_the_clamped_gated_activation(dtype, inter, limit):
     assert (np.abs(z[:, :inter]) > limit).any() and (z[:, inter:] < -limit).any()
 
 
+@pytest.mark.parametrize("rows, inter, k", [(1, 24, 64), (8, 70, 256), (16, 320, 256), (17, 48, 96), (32, 130, 512), (33, 24, 64)])
+def test_gated_product_with_biases_clamps_and_activation_in_its_last_step(rows, inter, k):
+    """Few bfloat16 rows: one kernel, bit-equal to the product followed by the activation's kernel
+    (33 rows: the two in turn, on both sides)."""
+    from mini_infer_amd import ops
+
+    rng = np.random.default_rng(rows * inter)
+    x = dev(rng.standard_normal((rows, k)).astype(np.float32), torch.bfloat16)
+    weight = dev((rng.standard_normal((2 * inter, k)) / np.sqrt(k) * 2.5).astype(np.float32), torch.bfloat16)
+    bias = dev(rng.standard_normal(2 * inter).astype(np.float32))
+    fused = ops.linear_clamped_glu(x, weight, bias, 1.3, 1.702)
+    in_turn = ops.clamped_glu(ops.linear(x, weight), bias, 1.3, 1.702)
+    assert torch.equal(fused, in_turn)
+    z = (x.double() @ weight.double().T).cpu().numpy() + bias.cpu().numpy()
+    g, u = np.minimum(z[:, :inter], 1.3), np.clip(z[:, inter:], -1.3, 1.3)
+    np.testing.assert_allclose(fused.float().cpu().numpy(), g / (1 + np.exp(-1.702 * g)) * (u + 1), rtol=0, atol=4e-2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channels, taps", [(10, 1), (70, 2), (256, 4), (33, 7)])
 def test_the_short_convolution_carries_each_requests_tail(dtype, channels, taps):
