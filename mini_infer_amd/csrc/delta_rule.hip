@@ -26,6 +26,7 @@
 #include <math.h>
 
 #define DELTA_MAX_TAPS 16
+#define SHORT_CONV_WALK_ROWS 64  // steps of at most this many rows: convolution and tail in one launch
 
 namespace {
 
@@ -83,6 +84,57 @@ __global__ __launch_bounds__(256) void short_conv_tail_kernel(const T* __restric
     const int at = n - back + j;
     mine[(int64_t)j * channels + c] = at >= 0 ? x[(int64_t)(first + at) * x_stride + c] : old[n + j];
   }
+}
+
+// Steps of few rows (decoded tokens, short portions): a thread walks the rows of one request on one
+// channel with the last taps-1 inputs in registers, and leaves them as the new tail: convolution
+// and tail in one launch.  The arithmetic is that of short_conv_kernel, term by term.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_walk_kernel(
+    const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w, T* __restrict__ tail, int64_t tail_stride,
+    const int* __restrict__ cu, const int* __restrict__ slots, T* __restrict__ y, int64_t y_stride, int channels, int taps,
+    int num_slots) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int first = cu[b], last = cu[b + 1];
+  if (last <= first) return;
+  const int slot = slots[b];
+  T* mine = tail + (int64_t)((slot < 0 || slot >= num_slots) ? num_slots : slot) * tail_stride;
+  const int back = taps - 1;
+  float window[DELTA_MAX_TAPS], wc[DELTA_MAX_TAPS];  // window[j]: the input `back - j` rows ago
+#pragma unroll
+  for (int j = 0; j < DELTA_MAX_TAPS; ++j) {
+    window[j] = j < back ? to_f32(mine[(int64_t)j * channels + c]) : 0.f;
+    wc[j] = j < taps ? w[(int64_t)c * taps + j] : 0.f;
+  }
+  for (int t = first; t < last; ++t) {
+    const float now = to_f32(x[(int64_t)t * x_stride + c]);
+    if constexpr (sizeof(T) == 4) {
+      double sum = 0.0;
+#pragma unroll
+      for (int j = 0; j < DELTA_MAX_TAPS; ++j)
+        if (j < back) sum = fma((double)wc[j], (double)window[j], sum);
+      sum = fma((double)w[(int64_t)c * taps + back], (double)now, sum);
+      y[(int64_t)t * y_stride + c] = (float)(sum / (1.0 + exp(-sum)));
+    } else {
+      float sum = 0.f;
+#pragma unroll
+      for (int j = 0; j < DELTA_MAX_TAPS; ++j)
+        if (j < back) sum = fmaf(wc[j], window[j], sum);
+      sum = fmaf(w[(int64_t)c * taps + back], now, sum);
+      y[(int64_t)t * y_stride + c] = from_f32<T>(sum * mi_logistic(sum));
+    }
+#pragma unroll
+    for (int j = 0; j < DELTA_MAX_TAPS - 1; ++j)
+      if (j + 1 < back) window[j] = window[j + 1];
+#pragma unroll
+    for (int j = 0; j < DELTA_MAX_TAPS; ++j)
+      if (j == back - 1) window[j] = now;
+  }
+#pragma unroll
+  for (int j = 0; j < DELTA_MAX_TAPS; ++j)
+    if (j < back) mine[(int64_t)j * channels + c] = from_f32<T>(window[j]);
 }
 
 // what a token's step needs beside q and k, made once per tile
@@ -368,6 +420,17 @@ extern "C" int mi_short_conv(int dtype, const void* x, int64_t x_stride, const f
   MI_REQUIRE(dtype == MI_F32 || dtype == MI_BF16, "short_conv: unknown dtype %d", dtype);
   if (num_tokens == 0 || num_requests == 0) return MI_OK;
   const int blocks = ceil_div(channels, 256);
+  if (num_tokens <= SHORT_CONV_WALK_ROWS) {
+    dim3 grid(blocks, num_requests);
+    if (dtype == MI_F32)
+      short_conv_walk_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, w, (float*)tail, tail_stride, cu, slots,
+                                                              (float*)y, y_stride, channels, taps, num_slots);
+    else
+      short_conv_walk_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_stride, w, (bf16_t*)tail, tail_stride, cu,
+                                                               slots, (bf16_t*)y, y_stride, channels, taps, num_slots);
+    MI_CHECK_LAUNCH("short_conv_walk");
+    return MI_OK;
+  }
   for (int first = 0; first < num_tokens; first += 65535) {
     dim3 grid(blocks, min(65535, num_tokens - first));
     if (dtype == MI_F32)

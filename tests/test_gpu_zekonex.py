@@ -143,7 +143,7 @@ def test_gated_product_with_biases_clamps_and_activation_in_its_last_step(rows, 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("channels, taps", [(10, 1), (70, 2), (256, 4), (33, 7)])
 def test_the_short_convolution_carries_each_requests_tail(dtype, channels, taps):
-    """Three steps over four requests of unequal length, among them portions shorter than the tail,
+    """Five steps over four requests of unequal length, among them portions shorter than the tail,
     a request that brings nothing, and one that starts later in a slot of its own."""
     from mini_infer_amd import ops
 
@@ -151,7 +151,8 @@ def test_the_short_convolution_carries_each_requests_tail(dtype, channels, taps)
     weight = (rng.standard_normal((channels, taps)) * 0.6).astype(np.float32)
     tails = torch.zeros((6, max(taps - 1, 0), channels), dtype=TORCH[dtype], device=DEV)
     plain = {slot: np.zeros((taps - 1, channels)) for slot in range(5)}
-    for step, lengths in enumerate([(1, 9, 0, 2), (2, 1, 5, 1), (40, 1, 1, 3)]):
+    # (steps of up to 64 rows run as one launch, a thread walking a request's rows; longer ones as two)
+    for step, lengths in enumerate([(1, 9, 0, 2), (2, 1, 5, 1), (80, 1, 1, 3), (1, 1, 0, 1), (30, 2, 70, 1)]):
         slots = [3, 0, 4, 1]
         x = rng.standard_normal((sum(lengths), channels + 5)).astype(np.float32)  # (the projection's rows are wider)
         cu = np.concatenate([[0], np.cumsum(lengths)])
