@@ -14,10 +14,10 @@
 //                     per column and silu(g).
 //
 // The state of a head lies in memory transposed and padded, [vdim][dim_pad].  Column j of S is
-// kept by 16 neighbouring lanes, each holding a run of its rows: a token costs a lane dim/16
+// kept by 16 or 32 neighbouring lanes, each holding a run of its rows: a token costs a lane a few
 // multiply-adds per pass and the partial sums meet through register moves between the lanes,
 // with no barrier inside a tile of tokens.  Columns are independent of one another, so a head's
-// work spreads over 16 * vdim threads however short the step.
+// work spreads over 16 or 32 times vdim threads however short the step.
 // Everything that enters the recurrence is float32 (the projections and the convolution's
 // outputs are read in the element type); in the 32-bit engine the scalar gates, the unit norms
 // and the read-out's norm are evaluated in 64-bit and rounded once.
@@ -142,8 +142,8 @@ struct TokenGates {
   float decay, write;
 };
 
-// Sum over the R neighbouring lanes that keep one column (R = 4, 8 or 16, inside a row of 16
-// lanes); every lane gets the total.  Lane exchanges inside a row are register moves (DPP):
+// Sum over the R neighbouring lanes that keep one column (R = 4, 8, 16 inside a row of 16
+// lanes, or 32: two rows); every lane gets the total.  Lane exchanges inside a row are register moves (DPP):
 // neighbours, pairs, then the mirror image inside 8 and inside 16 lanes, which after the first
 // two steps holds the other half's sum.
 template <int CTRL>
@@ -156,41 +156,49 @@ __device__ __forceinline__ float lanes_sum(float v) {
   v += dpp_move<0x4E>(v);  // quad_perm [2,3,0,1]
   if constexpr (R >= 8) v += dpp_move<0x141>(v);   // row_half_mirror
   if constexpr (R >= 16) v += dpp_move<0x140>(v);  // row_mirror
+  // (the other row of 16 inside 32 lanes: lane ^ 16, through the LDS crossbar without touching memory)
+  if constexpr (R >= 32) v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
   return v;
 }
 
-// 16 lanes keep a column of S, lane r of them its rows r * ROWS .. (r + 1) * ROWS - 1 (rows past
-// dim are zero and stay zero).  The columns of S do not meet in the recurrence, so a head's
-// columns are shared out among blocks: 256 threads keep 16 columns; thread = 16 * column + r.
-// The state of a head lies in memory as S transposed and padded, [vdim][16 * ROWS].  The read-outs
-// leave as float32 [tokens, heads * vdim]; their norm over a head's columns is the next kernel's.
+// R lanes (16 or 32) keep a column of S, lane r of them its rows r * ROWS .. (r + 1) * ROWS - 1
+// (rows past dim are zero and stay zero).  The columns of S do not meet in the recurrence, so a
+// head's columns are shared out among blocks: 256 threads keep 256 / R columns; thread = R *
+// column + r.  The state of a head lies in memory as S transposed and padded, [vdim][R * ROWS].
+// The read-outs leave as float32 [tokens, heads * vdim]; their norm over a head's columns is the
+// next kernel's.
 //
-// Tokens are taken 32 at a time.  A tile's rows are asked of memory while the tile before it is
-// worked on (they wait in registers); then 8 lanes a token make q and k unit vectors and put
-// them into LDS with the tile's values and gates, all 32 tokens at once; then the recurrence
-// walks the tile with LDS reads only, each token's operands read while the one before it is
-// worked on.  A step of the recurrence is 4 * ROWS multiply-adds a lane and two sums over 16
-// lanes by register moves.
-template <typename T, int ROWS>
+// Tokens are taken a tile (32, or 16) at a time.  A tile's rows are asked of memory while the
+// tile before it is worked on (they wait in registers); then a group of lanes per token makes q
+// and k unit vectors and puts them into LDS with the tile's values and gates, all tokens at once;
+// then the recurrence walks the tile with LDS reads only, each token's operands read while the
+// one before it is worked on.  A step of the recurrence is 4 * ROWS multiply-adds a lane and two
+// sums over R lanes by register moves.  Counters at heads of 128 x 128, 16 lanes a column: 100
+// vector instructions and 6 LDS reads a token and wave, one wave a SIMD, a token every 250 issue
+// turns.  32 lanes a column (half the work a wave, two waves a SIMD, twice the LDS reads a CU)
+// measured no faster, 961 against 912 us for 2,048 tokens, so 16 it is.
+template <typename T, int R, int ROWS>
 __global__ __launch_bounds__(256) void gated_delta_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, const T* __restrict__ proj, int64_t proj_stride, int col_b,
     int col_a, const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
     int64_t state_stride, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ readout,
     int heads, int kv_heads, int dim, int vdim, int chunks, int num_slots) {
   constexpr bool WIDE = sizeof(T) == 4;
-  constexpr int R = 16;            // lanes a column
   constexpr int PAD = R * ROWS;    // rows of S as kept: dim rounded up
   constexpr int COLS = 256 / R;    // columns of S this block keeps
-  constexpr int TILE = 32;         // tokens prepared together
-  constexpr int GROUP = 8;         // lanes that prepare one token
-  constexpr int EACH = PAD / GROUP;  // entries of a token's q (and k) row a lane prepares: two runs of ROWS
-  // (a lane's run of ROWS entries is followed by 4 unused ones: the runs that a 16-byte read of
-  // all lanes touches then lie in different banks)
-  constexpr int RUN = ROWS + 4;
+  // In LDS a lane's run of ROWS entries of q (and k) is followed by unused ones where runs of 32
+  // or 64 bytes would otherwise meet 2 or 4 to a bank in a 16-byte read of all lanes (runs of 16
+  // bytes lie side by side as they are).
+  constexpr int RUN = ROWS == 4 ? 4 : ROWS + 4;
   constexpr int LPAD = R * RUN;
+  constexpr int TILE = LPAD <= 192 ? 32 : 16;  // tokens prepared together (two tiles of LPAD floats each fit LDS)
+  constexpr int GROUP = 256 / TILE;            // lanes that prepare one token
+  constexpr int EACH = PAD / GROUP;            // entries of a token's q (and k) row a lane prepares
+  constexpr int VALUES = (TILE * COLS + 255) / 256;  // of the tile's values a thread fetches
+  static_assert(EACH % 4 == 0 && ROWS % 4 == 0, "entries are moved four at a time");
   __shared__ __align__(16) float q_tile[TILE * LPAD];
   __shared__ __align__(16) float k_tile[TILE * LPAD];
-  __shared__ float v_tile[TILE * COLS];
+  __shared__ float v_tile[VALUES * 256];
   __shared__ TokenGates gates[TILE];
 
   const int h = blockIdx.x / chunks, chunk = blockIdx.x % chunks, b = blockIdx.y;
@@ -218,10 +226,10 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(
   const float q_scale = 1.0f / sqrtf((float)dim);
   const float bias = dt_bias[h];
 
-  // what this thread prepares of a tile: token `mine_token` (8 lanes a token), entries
-  // sub * EACH .. of its q and k rows; and two of the tile's values
+  // what this thread prepares of a tile: token `mine_token` (GROUP lanes a token), entries
+  // sub * EACH .. of its q and k rows; and one or two of the tile's values
   const int mine_token = tid / GROUP, sub = tid % GROUP;
-  float q_raw[EACH], k_raw[EACH], v_raw[2], b_raw = 0.f, a_raw = 0.f;
+  float q_raw[EACH], k_raw[EACH], v_raw[VALUES], b_raw = 0.f, a_raw = 0.f;
   auto ask = [&](int t0, int nt) {
     const bool live = mine_token < nt;
     const T* row = qkv + (int64_t)(t0 + (live ? mine_token : 0)) * qkv_stride;
@@ -237,7 +245,7 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(
       a_raw = to_f32(p[col_a + h]);
     }
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < VALUES; ++n) {
       const int e = tid + n * 256, i = e / COLS, c = e % COLS;
       v_raw[n] = (i < nt && c < my_cols) ? to_f32(qkv[(int64_t)(t0 + i) * qkv_stride + v_col + c]) : 0.f;
     }
@@ -273,12 +281,13 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(
         q_inv = rsqrtf(lanes_sum<GROUP>(qq) + 1e-6f) * q_scale;
         k_inv = rsqrtf(lanes_sum<GROUP>(kk) + 1e-6f);
       }
-      // (a lane's entries are two runs of ROWS: runs 2 * sub and 2 * sub + 1 of the token's row)
-      float* q_at = q_tile + mine_token * LPAD + 2 * sub * RUN;
-      float* k_at = k_tile + mine_token * LPAD + 2 * sub * RUN;
+      // (entry d of a token's row lies at d + (d / ROWS) * (RUN - ROWS): runs of ROWS, each padded to RUN)
+      float* q_at = q_tile + mine_token * LPAD;
+      float* k_at = k_tile + mine_token * LPAD;
 #pragma unroll
       for (int e = 0; e < EACH; e += 4) {
-        const int at = e + (e / ROWS) * 4;
+        const int d = sub * EACH + e;
+        const int at = d + (d / ROWS) * (RUN - ROWS);
         *reinterpret_cast<float4*>(q_at + at) = make_float4(q_raw[e] * q_inv, q_raw[e + 1] * q_inv, q_raw[e + 2] * q_inv, q_raw[e + 3] * q_inv);
         *reinterpret_cast<float4*>(k_at + at) = make_float4(k_raw[e] * k_inv, k_raw[e + 1] * k_inv, k_raw[e + 2] * k_inv, k_raw[e + 3] * k_inv);
       }
@@ -297,8 +306,8 @@ __global__ __launch_bounds__(256) void gated_delta_kernel(
         }
         gates[mine_token] = gt;
       }
-      v_tile[tid] = v_raw[0];
-      v_tile[tid + 256] = v_raw[1];
+#pragma unroll
+      for (int n = 0; n < VALUES; ++n) v_tile[tid + n * 256] = v_raw[n];
     }
     __syncthreads();
     if (t0 + TILE < last) ask(t0 + TILE, min(TILE, last - t0 - TILE));  // (waits in registers through the steps below)
@@ -393,13 +402,12 @@ __global__ __launch_bounds__(256) void delta_readout_norm_kernel(const float* __
   }
 }
 
-// How a head's state is kept for these sizes: 16 lanes a column, ROWS rows a lane (4, 8 or 16: the
-// next of them that holds dim / 16).
+// How a head's state is kept for these sizes: 16 lanes a column, 4, 8 or 16 rows a lane (the next of
+// them that holds dim / 16).
 static void delta_layout(int dim, int vdim, int* lanes, int* rows) {
   (void)vdim;
   *lanes = 16;
-  const int need = ceil_div(dim, 16);
-  *rows = need <= 4 ? 4 : (need <= 8 ? 8 : 16);
+  *rows = dim <= 64 ? 4 : (dim <= 128 ? 8 : 16);
 }
 
 }  // namespace
@@ -495,14 +503,14 @@ extern "C" int mi_gated_delta(int dtype, const void* qkv, int64_t qkv_stride, co
   const int cols = 256 / lanes, chunks = ceil_div(vdim, cols);
   MI_REQUIRE((int64_t)heads * chunks <= 2147483647, "gated_delta: too many heads");
   dim3 grid(heads * chunks, num_requests);
-#define MI_DELTA_LAUNCH(T, ROWS)                                                                                 \
-  gated_delta_kernel<T, ROWS><<<grid, 256, 0, stream>>>(                                                         \
+#define MI_DELTA_LAUNCH(T, RR, ROWS)                                                                             \
+  gated_delta_kernel<T, RR, ROWS><<<grid, 256, 0, stream>>>(                                                     \
       (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, col_b, col_a, a_log, dt_bias, state, state_stride, \
       cu, slots, readout, heads, kv_heads, dim, vdim, chunks, num_slots)
-#define MI_DELTA_LANES(T)                     \
-  if (rows == 4) MI_DELTA_LAUNCH(T, 4);       \
-  else if (rows == 8) MI_DELTA_LAUNCH(T, 8);  \
-  else MI_DELTA_LAUNCH(T, 16);
+#define MI_DELTA_LANES(T)                          \
+  if (rows == 4) MI_DELTA_LAUNCH(T, 16, 4);        \
+  else if (rows == 8) MI_DELTA_LAUNCH(T, 16, 8);   \
+  else MI_DELTA_LAUNCH(T, 16, 16);
   if (dtype == MI_F32) { MI_DELTA_LANES(float) }
   else { MI_DELTA_LANES(bf16_t) }
 #undef MI_DELTA_LANES

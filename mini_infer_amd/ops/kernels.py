@@ -1622,11 +1622,9 @@ def short_conv(
 
 def delta_state_shape(heads: int, dim: int, vdim: int) -> tuple[int, int, int]:
     """How `gated_delta` lays a request's state out: per head S transposed, [vdim][padded dim].
-    A column is kept by 16 neighbouring lanes, each holding 4, 8 or 16 rows: the padded dim is
-    their product (the kernel checks it)."""
-    need = -(-dim // 16)
-    rows = 4 if need <= 4 else (8 if need <= 8 else 16)
-    return (heads, vdim, 16 * rows)
+    A column is kept by 16 neighbouring lanes with 4, 8 or 16 rows each: the padded dim is their
+    product (the kernel checks it)."""
+    return (heads, vdim, 64 if dim <= 64 else (128 if dim <= 128 else 256))
 
 
 def gated_delta(
