@@ -53,7 +53,7 @@ class GQAttention(Mixer):
     ) -> None:
         """`v_head_dim`: value heads of another width than the query and key heads (`head_dim`).
         `sink_logit`: the softmax's denominator gets one more term exp(sink_logit), a sink that
-        takes weight off the keys and carries no value (0.0: "one added to the denominator")."""
+        takes weight off the keys and carries no value (0.0: the denominator grows by exp(0) = 1)."""
         super().__init__(dtype, device)
         if num_heads % num_kv_heads != 0:
             raise ValueError(f"num_heads={num_heads} is not a multiple of num_kv_heads={num_kv_heads}")
