@@ -472,6 +472,32 @@ def test_greedy_generation_through_llm_and_the_scheduler(folders, name):
     llm.runner.cache.check()
 
 
+def test_the_command_line_writes_random_weights_and_generates_greedily_and_by_seeded_sampling(tmp_path, capsys):
+    """`random-weights` from a config.json, then `generate`: greedy twice the same, sampled with one seed
+    twice the same and (at this temperature) different from greedy."""
+    from mini_infer_amd.__main__ import main
+
+    cfg, block = tz.CONFIGS["A"]
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    assert main(["random-weights", "--config", str(tmp_path / "config.json"), "--seed", "3", "--out", str(tmp_path / "m"),
+                 "--std", "0.3", "--norm-jitter", "0.1"]) == 0
+    capsys.readouterr()
+
+    def generate(*extra):
+        assert main(["generate", "--model", str(tmp_path / "m"), "--prompt-ids", "5 9 100 3 77", "--prompt-ids", "1,2",
+                     "--max-tokens", "12", "--num-blocks", "16", "--block-size", str(block), "--max-concurrent", "2",
+                     "--ignore-eos", *extra]) == 0
+        lines = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+        assert [line["prompt_tokens"] for line in lines] == [5, 2] and all(len(line["tokens"]) == 12 for line in lines)
+        return [line["tokens"] for line in lines]
+
+    greedy = generate()
+    assert generate() == greedy
+    sampled = generate("--temperature", "1.5", "--top-k", "40", "--top-p", "0.95", "--seed", "11")
+    assert generate("--temperature", "1.5", "--top-k", "40", "--top-p", "0.95", "--seed", "11") == sampled
+    assert sampled != greedy and all(0 <= t < cfg["vocab"] for tokens in sampled for t in tokens)
+
+
 def test_the_replay_program_runs_a_trace_of_this_design(folders, tmp_path):
     from mini_infer_amd.engine import replay, trace
 
