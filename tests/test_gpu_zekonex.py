@@ -472,6 +472,37 @@ def test_greedy_generation_through_llm_and_the_scheduler(folders, name):
     llm.runner.cache.check()
 
 
+def test_a_norm_that_knows_no_stream_update_is_handed_the_finished_sum(folders):
+    """The parallel block leaves its add to the next norm as an update not made yet.  `rms_norm` makes it
+    in its own launch; a norm of another kind (here the one-gain norm as final norm) gets the finished
+    sum instead.  With a weight that is the gain in every column the two models are one function."""
+    import dataclasses
+
+    from mini_infer_amd.engine import ModelRunner, StepEntry
+    from mini_infer_amd.models.decoder import DecoderModel
+    from mini_infer_amd.models.zekonex import ZekonexConfig, zekonex_spec
+    from mini_infer_amd.weights.loader import load_state_dict
+
+    cfg, block, weights, _ = folders["A"]
+    spec = zekonex_spec(ZekonexConfig.from_dict(cfg))
+    one_gain = dataclasses.replace(spec, final_norm={"kind": "scalar_rms_norm", "hidden_size": cfg["width"],
+                                                     "eps": cfg["norm"]["eps"], "name": "norm"})
+    tensors = {k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in weights.items()}
+    tokens = tz.random_tokens(cfg, 37, seed=8)
+    got = []
+    for model_spec, final in ((spec, torch.full((cfg["width"],), 0.75)), (one_gain, torch.tensor(0.75))):
+        model = DecoderModel(model_spec, torch.float32, DEV)
+        load_state_dict(model, dict(tensors, **{"final.norm": final}))
+        runner = ModelRunner(model, None, num_blocks=4, block_size=block, max_concurrent=1)
+        first = runner.step([StepEntry("r", tokens[:30], list(range(30)))]).cpu().numpy()
+        rest = [runner.step([StepEntry("r", [t], [0])]).cpu().numpy() for t in tokens[30:]]
+        got.append(np.concatenate([first, *rest]))
+    np.testing.assert_allclose(got[1], got[0], rtol=0, atol=2e-5)
+    wide = {k: v.astype(np.float64) for k, v in weights.items()}
+    wide["final.norm"] = np.full(cfg["width"], 0.75)
+    ru.assert_close(got[0], pz.logits(cfg, wide, tokens), "float32", "weight of one value")
+
+
 def test_the_command_line_writes_random_weights_and_generates_greedily_and_by_seeded_sampling(tmp_path, capsys):
     """`random-weights` from a config.json, then `generate`: greedy twice the same, sampled with one seed
     twice the same and (at this temperature) different from greedy."""
